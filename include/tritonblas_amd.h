@@ -1,0 +1,197 @@
+/*
+ * tritonblas_amd — C ABI of the MI355X (gfx950) GEMM library.
+ *
+ * The reference (ROCm/tritonBLAS) has no FFI: its boundary is a Python API whose launchers start
+ * Triton kernels.  Each entry point below replaces one of those launch sites; the Python package
+ * binds them with ctypes.  All pointers are borrowed device pointers (the caller keeps the memory
+ * alive until the stream has run the kernel), the library allocates nothing on the device, every
+ * launch is asynchronous on the given stream, and errors are negative status codes (no exceptions,
+ * no abort).
+ */
+#ifndef TRITONBLAS_AMD_H
+#define TRITONBLAS_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TB_ABI_VERSION 1
+
+/* ---- status codes --------------------------------------------------------------------------- */
+enum {
+  TB_OK = 0,
+  TB_ERR_NULL_POINTER = -1,
+  TB_ERR_BAD_SHAPE = -2,        /* the reference's  assert "Incompatible Dimensions"  (matmul.py:81) */
+  TB_ERR_BAD_DTYPE = -3,
+  TB_ERR_BAD_LAYOUT = -4,       /* strides this kernel family cannot address                        */
+  TB_ERR_BAD_TILE = -5,         /* (block_m, block_n, block_k) is not a built kernel variant        */
+  TB_ERR_WORKSPACE = -6,        /* workspace missing or too small for the requested schedule        */
+  TB_ERR_BAD_SCHEDULE = -7,     /* grid larger than what can be co-resident, bad group table, ...   */
+  TB_ERR_LAUNCH = -8,           /* the HIP runtime refused the launch                               */
+  TB_ERR_NO_DEVICE = -9,
+  TB_ERR_BAD_ARGUMENT = -10
+};
+
+/* ---- element types -------------------------------------------------------------------------- */
+enum {
+  TB_F16 = 0,
+  TB_BF16 = 1,
+  TB_FP8_E4M3 = 2,  /* OCP e4m3fn                                                  */
+  TB_FP4_E2M1 = 3,  /* two codes per byte, low nibble = even k (utils.py:585-587) */
+  TB_F32 = 4        /* output / bias / quantiser input only                        */
+};
+
+/* ---- schedules ------------------------------------------------------------------------------ */
+enum {
+  TB_SCHED_PERSISTENT = 0,    /* data parallel, one tile per workgroup   (matmul.py:160-198)        */
+  TB_SCHED_WORK_STEALING = 1, /* atomic tile queues per XCD x slot       (matmul.py:112-159)        */
+  TB_SCHED_STREAMK = 2        /* data parallel tiles + Stream-K tail     (matmul.py:202-366)        */
+};
+
+/* ---- hardware descriptor (replaces origami.get_hardware_for_device, origami.py:166) --------- */
+typedef struct tb_hw {
+  int32_t n_cu;          /* compute units                                   */
+  int32_t num_xcd;       /* accelerator complex dies (one L2 each)          */
+  int32_t cu_per_xcd;
+  int32_t lds_bytes;     /* LDS per CU                                      */
+  int32_t l2_bytes;      /* L2 per XCD                                      */
+  int32_t clock_khz;     /* peak engine clock                               */
+  int32_t mem_clock_khz;
+  int32_t wave_size;
+  double hbm_gbps;       /* peak HBM bandwidth, GB/s                        */
+  char arch[32];         /* "gfx950"                                        */
+} tb_hw;
+
+/* Fills *out for HIP device `device`; with device < 0 (or no GPU present and device == -1) fills
+ * the MI355X defaults so that the analytical selector can run on a machine without a GPU. */
+int tb_device_info(int device, tb_hw* out);
+
+/* ---- analytical selector (replaces origami.select_config / select_workgroup_mapping and
+ *      OrigamiMatmulSelector._compute_sk_grid / _select_ws_params, origami.py:232-286,349-416) --- */
+typedef struct tb_problem {
+  int64_t m, n, k;
+  int32_t a_type, b_type, c_type;
+  int32_t a_k_contiguous;   /* 1: A is (m,k) with unit k stride   */
+  int32_t b_k_contiguous;   /* 1: B is stored (n,k) with unit k stride */
+  int32_t streamk;          /* caller intends enable_streamk=True  */
+  int32_t num_groups;       /* >0: grouped (MoE) problem, m = total rows */
+} tb_problem;
+
+typedef struct tb_selection {
+  int32_t block_m, block_n, block_k;
+  int32_t group_m;            /* GROUP_M swizzle height (origami.py:286)                  */
+  int32_t num_xcds;           /* XCD remap modulus (selector.num_sms, origami.py:330)     */
+  int32_t occupancy;          /* workgroups per CU the variant was sized for              */
+  int32_t num_stages;
+  int32_t sk_grid;            /* Stream-K grid (origami.py:349)                           */
+  int32_t counters_per_xcd;   /* work-stealing slots per XCD (origami.py:266-284)         */
+  int32_t lds_bytes;          /* LDS the chosen variant allocates                         */
+  double est_compute_us, est_memory_us, est_total_us;
+} tb_selection;
+
+int tb_select(const tb_problem* problem, const tb_hw* hw, tb_selection* out);
+
+/* Number of built tile variants for (a_type); fills up to `cap` (block_m, block_n, block_k) triples. */
+int tb_list_tiles(int32_t a_type, int32_t* triples, int32_t cap);
+
+/* ---- GEMM ----------------------------------------------------------------------------------- */
+typedef struct tb_gemm_desc {
+  uint32_t struct_bytes;      /* sizeof(tb_gemm_desc), checked                                       */
+  int32_t a_type, b_type, c_type, bias_type;
+  int64_t m, n, k;            /* logical sizes: A (m,k), B (k,n), C (m,n)                           */
+  int64_t a_stride_m, a_stride_k;   /* element strides (torch's a.stride())                         */
+  int64_t b_stride_k, b_stride_n;
+  int64_t c_stride_m, c_stride_n;
+  const void* a;
+  const void* b;
+  void* c;
+  const float* a_scale;       /* per row of A (m), or NULL      (matmul_a8w8_lt, matmul.py:380)      */
+  const float* b_scale;       /* per column of B (n), or NULL                                        */
+  const void* bias;           /* per column (n), or NULL        (addmm, matmul.py:727)               */
+  int64_t bias_stride;
+  int32_t block_m, block_n, block_k;  /* tile variant, from tb_select; 0 = let the library select    */
+  int32_t group_m, num_xcds;
+  int32_t schedule;           /* TB_SCHED_*                                                         */
+  int32_t grid;               /* Stream-K / work-stealing grid; 0 = default                         */
+  int32_t counters_per_xcd;
+  void* workspace;            /* tb_workspace_bytes() bytes, zero-initialised once by the caller     */
+  size_t workspace_bytes;
+  uint32_t epoch;             /* Stream-K: must differ from the previous launch on this workspace    */
+  uint32_t spin_limit;        /* Stream-K: bound on flag polls per wait; 0 = default                 */
+} tb_gemm_desc;
+
+/* C = cast((A @ B) * a_scale[:,None] * b_scale[None,:] + bias[None,:]), fp32 accumulate.
+ * Replaces persistent_matmul_lt / streamk_matmul_lt (matmul.py:69-366). */
+int tb_gemm(const tb_gemm_desc* desc, void* stream);
+
+/* Bytes of workspace tb_gemm needs for this descriptor (0 for the persistent schedule). */
+size_t tb_workspace_bytes(const tb_gemm_desc* desc);
+
+/* ---- MXFP4 GEMM (replaces matmul_fp4, matmul.py:519-625) ------------------------------------- */
+typedef struct tb_gemm_fp4_desc {
+  uint32_t struct_bytes;
+  int32_t c_type;
+  int64_t m, n, k;            /* k = unpacked element count, multiple of 32                          */
+  const void* a;              /* (m, k/2) bytes, k-contiguous                                        */
+  const void* b;              /* (n, k/2) bytes, k-contiguous                                        */
+  void* c;
+  int64_t a_stride_m, b_stride_n;     /* row strides in bytes                                        */
+  int64_t c_stride_m, c_stride_n;
+  const void* a_scales;       /* (m, k/32) E8M0 bytes                                                */
+  const void* b_scales;       /* (n, k/32) E8M0 bytes                                                */
+  int64_t a_scales_stride_m, a_scales_stride_k;
+  int64_t b_scales_stride_n, b_scales_stride_k;
+  int32_t block_m, block_n, block_k;  /* 0 = select                                                  */
+  int32_t group_m, num_xcds;
+} tb_gemm_fp4_desc;
+
+int tb_gemm_fp4(const tb_gemm_fp4_desc* desc, void* stream);
+
+/* ---- grouped (MoE) FP8 GEMM — no counterpart in the reference -------------------------------- */
+typedef struct tb_grouped_gemm_desc {
+  uint32_t struct_bytes;
+  int32_t c_type;
+  int64_t m_total, n, k;      /* rows over all experts, per-expert weight (n,k)                      */
+  int32_t num_groups;
+  const void* a;              /* (m_total, k) e4m3, rows sorted by expert, k-contiguous              */
+  const void* w;              /* (num_groups, n, k) e4m3, k-contiguous                               */
+  void* c;                    /* (m_total, n)                                                        */
+  int64_t a_stride_m, w_stride_g, w_stride_n;
+  int64_t c_stride_m, c_stride_n;
+  const float* a_scale;       /* (m_total)                                                           */
+  const float* w_scale;       /* (num_groups, n) contiguous                                          */
+  const int32_t* group_offsets; /* device int32[num_groups+1], offsets[0]=0, offsets[g]=m_total     */
+  int32_t block_m, block_n, block_k;
+  int32_t group_m, num_xcds;
+} tb_grouped_gemm_desc;
+
+int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* desc, void* stream);
+
+/* ---- MXFP4 quantisation (replaces dynamic_mxfp4_quant, utils.py:743-789), optionally preceded
+ *      by a 32-point blockwise Hadamard rotation along k (no counterpart in the reference) ------- */
+typedef struct tb_quant_desc {
+  uint32_t struct_bytes;
+  int32_t x_type;             /* TB_BF16, TB_F16 or TB_F32                                           */
+  int64_t m, n;               /* n multiple of 32                                                    */
+  const void* x;
+  int64_t x_stride_m;         /* elements; unit stride along n                                       */
+  void* codes;                /* (m, n/2) bytes                                                      */
+  int64_t codes_stride_m;
+  void* scales;               /* (m, n/32) bytes                                                     */
+  int64_t scales_stride_m;
+  int32_t hadamard;           /* 1: rotate each block of 32 by H32/sqrt(32) first                    */
+} tb_quant_desc;
+
+int tb_hadamard_mxfp4_quant(const tb_quant_desc* desc, void* stream);
+
+/* ---- misc ----------------------------------------------------------------------------------- */
+const char* tb_status_string(int status);
+int tb_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITONBLAS_AMD_H */

@@ -1,0 +1,85 @@
+"""GEMM oracles: fp32 CPU ``torch.matmul`` of the (dequantised) operands, then the fused epilogue.
+
+Test infrastructure: see ``oracle/__init__.py``.
+
+These are the reference's own oracles restated:
+  * fp16/bf16: ``torch.matmul`` / ``torch.mm``   tests/test_matmul_correctness.py:44, tests/test_matmul_lt.py:60
+  * a8w8:      fp32 matmul * (sa[:,None]*sb[None,:]) (+bias) -> clamp for fp8 out -> cast
+               tests/test_matmul_a8w8_lt.py:11-38, benchmarks/tritonblas_matmul.py:62-76
+  * MXFP4:     LUT x E8M0 dequant, ``torch.mm(x, w.T)``   tests/test_matmul_fp4.py:20-46
+  * FP8 per-channel quantisation recipe   include/tritonblas/utils.py:340-377
+The grouped (MoE) GEMM has no reference code; it is the concatenation of per-expert a8w8 closed forms.
+"""
+import numpy as np
+import torch
+
+from . import mxfp4
+
+
+def quantize_per_channel_fp8(x: torch.Tensor, axis: int, dtype=torch.float8_e4m3fn, min_scale: float = 1e-8):
+    """include/tritonblas/utils.py:340-377: amax -> scale = amax/448 -> q = (x * (1/scale)).to(fp8)."""
+    base = x.to(torch.float32)
+    max_abs = torch.clamp(base.abs().amax(dim=axis, keepdim=True), min=min_scale)
+    scale = max_abs / torch.finfo(dtype).max
+    inv = 1.0 / scale
+    q = (base * inv).to(dtype)
+    return q, scale.squeeze(axis).to(torch.float32)
+
+
+def ref_gemm(a: torch.Tensor, b: torch.Tensor, out_dtype=None, a_scale=None, b_scale=None, bias=None):
+    """C = cast((fp32(A) @ fp32(B)) * (sa[:,None]*sb[None,:]) + bias[None,:]).
+
+    a: (M, K), b: (K, N), any strides, any float dtype that converts to fp32 (incl. float8_e4m3fn).
+    Epilogue order follows tests/test_matmul_a8w8_lt.py:11-38; the bias is per output *column*
+    (include/tritonblas/kernels/stages/matrix_view.py:194-208, tests/test_addmm_correctness.py:35)."""
+    acc = torch.matmul(a.to(torch.float32), b.to(torch.float32))
+    if a_scale is not None and b_scale is not None:
+        acc = acc * (a_scale.to(torch.float32)[:, None] * b_scale.to(torch.float32)[None, :])
+    if bias is not None:
+        acc = acc + bias.to(torch.float32)[None, :]
+    if out_dtype is None:
+        out_dtype = a.dtype
+    if out_dtype in (torch.float8_e4m3fn,):
+        mx = torch.finfo(out_dtype).max
+        acc = torch.clamp(acc, -mx, mx)
+    return acc.to(out_dtype)
+
+
+def ref_gemm_fp4(a_codes, b_codes, a_scales, b_scales, out_dtype=torch.bfloat16, return_fp32=False):
+    """a_codes (M, K/2) u8, b_codes (N, K/2) u8, scales (M|N, K/32) u8 -> (M, N).
+
+    tests/test_matmul_fp4.py:20-46."""
+    A = torch.from_numpy(mxfp4.dequant(_np(a_codes), _np(a_scales)))
+    B = torch.from_numpy(mxfp4.dequant(_np(b_codes), _np(b_scales)))
+    acc = torch.mm(A, B.T)
+    return acc if return_fp32 else acc.to(out_dtype)
+
+
+def ref_grouped_gemm_fp8(a_q, w_q, a_scale, w_scale, offsets, out_dtype=torch.bfloat16, return_fp32=False):
+    """a_q (M, K) fp8 rows sorted by expert; w_q (E, N, K) fp8; a_scale (M,), w_scale (E, N);
+    offsets int (E+1,) row boundaries.  Rows of expert e: C[o[e]:o[e+1]] = a8w8 closed form with W[e]."""
+    E, N, K = w_q.shape
+    M = a_q.shape[0]
+    out = torch.zeros(M, N, dtype=torch.float32)
+    off = [int(v) for v in offsets]
+    for e in range(E):
+        lo, hi = off[e], off[e + 1]
+        if hi <= lo:
+            continue
+        acc = torch.matmul(a_q[lo:hi].to(torch.float32), w_q[e].to(torch.float32).T)
+        out[lo:hi] = acc * (a_scale[lo:hi].to(torch.float32)[:, None] * w_scale[e].to(torch.float32)[None, :])
+    return out if return_fp32 else out.to(out_dtype)
+
+
+def rel_fro_error(got: torch.Tensor, want: torch.Tensor) -> float:
+    """||got - want||_F / ||want||_F in fp64 (the parity measure the tolerances are stated in)."""
+    g = got.detach().to("cpu", torch.float64)
+    w = want.detach().to("cpu", torch.float64)
+    den = torch.linalg.norm(w).item()
+    return torch.linalg.norm(g - w).item() / (den if den > 0 else 1.0)
+
+
+def _np(t):
+    if isinstance(t, torch.Tensor):
+        return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+    return np.asarray(t, dtype=np.uint8)

@@ -1,0 +1,109 @@
+"""Integer tile-schedule functions restated from the reference's device code (pure Python ints).
+
+Test infrastructure: see ``oracle/__init__.py``.
+"""
+
+
+def cdiv(a, b):
+    return -(-a // b)
+
+
+def chiplet_transform(pid, num_workgroups, num_xcds):
+    """include/tritonblas/kernels/stages/indexing/pid_transforms.py:6-16."""
+    xcd = pid % num_xcds
+    pos_in_xcd = pid // num_xcds
+    min_per_xcd = num_workgroups // num_xcds
+    extra = num_workgroups % num_xcds
+    return xcd * min_per_xcd + min(xcd, extra) + pos_in_xcd
+
+
+def chiplet_transform_chunked(pid, num_workgroups, num_xcds, chunk_size):
+    """include/tritonblas/kernels/stages/indexing/pid_transforms.py:20-38 (note the strict '>')."""
+    block = num_xcds * chunk_size
+    if pid > (num_workgroups // block) * block:
+        return pid
+    local_pid = pid // num_xcds
+    chunk_idx = local_pid // chunk_size
+    pos_in_chunk = local_pid % chunk_size
+    xcd = pid % num_xcds
+    return chunk_idx * block + xcd * chunk_size + pos_in_chunk
+
+
+def tile_coords(tile_id, num_pid_m, num_pid_n, group_m):
+    """GROUP_M swizzle: include/tritonblas/kernels/stages/schedule.py:124-145."""
+    num_pid_in_group = group_m * num_pid_n
+    group_id = tile_id // num_pid_in_group
+    first_pid_m = group_id * group_m
+    gsz = min(num_pid_m - first_pid_m, group_m)
+    pid_m = first_pid_m + ((tile_id % num_pid_in_group) % gsz)
+    pid_n = (tile_id % num_pid_in_group) // gsz
+    return pid_m, pid_n
+
+
+def launch_chunk_size(group_m, total_programs, num_xcds):
+    """include/tritonblas/matmul.py:105-110."""
+    chunk = group_m * group_m
+    if num_xcds > 0:
+        chunk = min(chunk, max(1, total_programs // num_xcds))
+    return chunk
+
+
+def streamk_partition(total_tiles, grid):
+    """include/tritonblas/matmul.py:238-241: tiles handled by the Stream-K tail."""
+    return total_tiles % grid if grid > 0 else 0
+
+
+def streamk_iter_range(pid, grid, total_tiles, sk_tiles, iters_per_tile):
+    """include/tritonblas/kernels/stages/schedule.py:190-223 / streamk_gemm.py:175-181."""
+    full = total_tiles - sk_tiles
+    total_sk_iters = sk_tiles * iters_per_tile
+    q, r = divmod(total_sk_iters, grid)
+    start = full * iters_per_tile + pid * q + min(pid, r)
+    end = full * iters_per_tile + (pid + 1) * q + min(pid + 1, r)
+    return start, end
+
+
+def streamk_segments(pid, grid, total_tiles, sk_tiles, iters_per_tile):
+    """Segments [(tile, k_first, k_last_exclusive, is_tile_start)] one workgroup walks in its Stream-K
+    range: include/tritonblas/kernels/streamk_gemm.py:184-187."""
+    start, last = streamk_iter_range(pid, grid, total_tiles, sk_tiles, iters_per_tile)
+    out = []
+    while start < last:
+        rem = start % iters_per_tile
+        end = min(start + (iters_per_tile - rem), last)
+        tile = start // iters_per_tile
+        out.append((tile, rem, rem + (end - start), rem == 0))
+        start = end
+    return out
+
+
+def ws_slot_range(pid, total_tiles, num_xcds, counters_per_xcd):
+    """Flat work-stealing queue a workgroup pulls from:
+    include/tritonblas/kernels/persistent_gemm_work_stealing.py:296-314.
+    Returns (counter_index, first_tile, bound)."""
+    xcd = pid % num_xcds
+    tiles_per_xcd = cdiv(total_tiles, num_xcds)
+    slot = (pid // num_xcds) % counters_per_xcd
+    xcd_base = xcd * tiles_per_xcd
+    xcd_end = min(xcd_base + tiles_per_xcd, total_tiles)
+    tiles_this_xcd = max(xcd_end - xcd_base, 0)
+    tiles_per_slot = cdiv(tiles_this_xcd, counters_per_xcd)
+    slot_base = slot * tiles_per_slot
+    slot_end = min(slot_base + tiles_per_slot, tiles_this_xcd)
+    return xcd * counters_per_xcd + slot, xcd_base + slot_base, max(slot_end - slot_base, 0)
+
+
+def grouped_tile_lookup(tile_id, offsets, block_m, tiles_n):
+    """Grouped (MoE) tile table: experts in order, each contributes cdiv(rows_e, block_m) * tiles_n
+    tiles, m-block fastest.  Returns (expert, m_block, n_block) or None past the end.  New work, no
+    reference counterpart."""
+    acc = 0
+    for e in range(len(offsets) - 1):
+        rows = offsets[e + 1] - offsets[e]
+        mb = cdiv(rows, block_m) if rows > 0 else 0
+        cnt = mb * tiles_n
+        if tile_id < acc + cnt:
+            local = tile_id - acc
+            return e, local % mb, local // mb
+        acc += cnt
+    return None

@@ -1,0 +1,285 @@
+"""GPU parity tests of the GEMM entry points against the CPU oracle (all launches go through the
+C ABI).  Tolerances: relative Frobenius error <= 1e-3 for fp16/bf16 and <= 1e-2 for FP8/MXFP4,
+measured against the oracle's fp32 GEMM of the (dequantised) operands rounded to the output type
+the same way the kernel's epilogue rounds."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import DTYPES, EDGE_CASE_DIMS, SKINNY_DIMS, STANDARD_DIMS
+from oracle import gemm as OG
+from oracle import inputs as OI
+from oracle import mxfp4 as OM
+
+pytestmark = pytest.mark.gpu
+
+TOL_16 = 1e-3
+TOL_Q = 1e-2
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _layout(x_cpu, trans):
+    """Reference convention (utils.py:495-505): "T" keeps the logical shape contiguous, "N" stores
+    the transpose and hands out a view."""
+    x = x_cpu.cuda()
+    if trans == "T":
+        return x.contiguous()
+    return x.T.contiguous().T
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _check(c_gpu, want_fp32, out_dtype, tol):
+    want = want_fp32.to(out_dtype)
+    err = OG.rel_fro_error(c_gpu.float(), want.float())
+    assert err <= tol, f"relative Frobenius error {err:.3e} > {tol}"
+    return err
+
+
+@pytest.mark.parametrize("m,n,k", STANDARD_DIMS + EDGE_CASE_DIMS + SKINNY_DIMS)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("transA,transB", [("T", "T"), ("N", "N"), ("T", "N"), ("N", "T")])
+def test_matmul_16bit(m, n, k, dtype, transA, transB):
+    import tritonblas_amd as tb
+    _say(f"matmul {m}x{n}x{k} {dtype} {transA}{transB}")
+    a_cpu, b_cpu = _rand((m, k), dtype, 0, 0.5), _rand((k, n), dtype, 10000, 0.5)
+    a, b = _layout(a_cpu, transA), _layout(b_cpu, transB)
+    c = tb.matmul(a, b)
+    assert c.shape == (m, n) and c.dtype == dtype
+    _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32), dtype, TOL_16)
+
+
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (512, 768, 320), (300, 200, 192), (257, 129, 64)])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tile", [(256, 256, 64), (128, 128, 64), (64, 64, 64)])
+def test_every_16bit_tile_variant(m, n, k, dtype, tile):
+    """Forces each built tile through matmul_lt (the selector would otherwise pick one)."""
+    import tritonblas_amd as tb
+    _say(f"matmul_lt {m}x{n}x{k} {dtype} tile={tile}")
+    a_cpu, b_cpu = _rand((m, k), dtype, 1, 0.5), _rand((k, n), dtype, 10001, 0.5)
+    want = OG.ref_gemm(a_cpu, b_cpu, torch.float32)
+    for ta, tb_ in [("T", "T"), ("T", "N"), ("N", "T"), ("N", "N")]:
+        a, b = _layout(a_cpu, ta), _layout(b_cpu, tb_)
+        sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device)
+        sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = tile
+        c = torch.zeros(m, n, dtype=dtype, device="cuda")
+        out = tb.matmul_lt(a, b, c, sel, None)
+        assert out is c
+        _check(c.cpu(), want, dtype, TOL_16)
+
+
+def test_config1_fp16_1024():
+    import tritonblas_amd as tb
+    a_cpu, b_cpu = OI.c1_fp16()
+    sel = tb.OrigamiMatmulSelector(1024, 1024, 1024, torch.float16, torch.float16, torch.float16, torch.device("cuda"))
+    cfg = tb.matmul_preamble(sel)
+    c = torch.empty(1024, 1024, dtype=torch.float16, device="cuda")
+    tb.matmul_lt(a_cpu.cuda(), b_cpu.cuda(), c, sel, cfg)
+    err = _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32), torch.float16, TOL_16)
+    _say(f"config 1 fp16 1024^3 rel fro err {err:.2e}")
+
+
+def test_out_semantics_and_autograd():
+    import tritonblas_amd as tb
+    a = _rand((64, 128), torch.bfloat16, 3).cuda()
+    b = _rand((128, 32), torch.bfloat16, 4).cuda()
+    out = torch.empty(64, 32, dtype=torch.bfloat16, device="cuda")
+    assert tb.matmul(a, b, out=out) is None
+    assert torch.equal(out, tb.matmul(a, b))
+    with pytest.raises(RuntimeError, match="differentiation"):
+        tb.matmul(a.clone().requires_grad_(), b, out=out)
+    with pytest.raises(AssertionError):
+        tb.matmul(a, a)
+    a32, b32 = a.float().requires_grad_(), b.float().requires_grad_()
+    (a32 @ b32).sum().backward()
+    ag, bg = a.clone().requires_grad_(), b.clone().requires_grad_()
+    tb.matmul(ag, bg).sum().backward()
+    assert OG.rel_fro_error(ag.grad.float().cpu(), a32.grad.cpu()) < 1e-2
+    assert OG.rel_fro_error(bg.grad.float().cpu(), b32.grad.cpu()) < 1e-2
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 256, 512), (15, 17, 512), (512, 1024, 768)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_addmm_column_bias(m, n, k, dtype):
+    import tritonblas_amd as tb
+    a_cpu, b_cpu, bias_cpu = _rand((m, k), dtype, 5, 0.5), _rand((k, n), dtype, 6, 0.5), _rand((n,), dtype, 7)
+    c = tb.addmm(bias_cpu.cuda(), a_cpu.cuda(), b_cpu.cuda())
+    _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32, bias=bias_cpu), dtype, TOL_16)
+
+
+# ---- FP8 a8w8 -----------------------------------------------------------------------------------
+def _a8w8_case(m, n, k, seed=2):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(n, k, generator=torch.Generator().manual_seed(seed + 10000)).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    bq, sb = OG.quantize_per_channel_fp8(w.T, axis=0)   # B = (K, N) view of the (N, K) weight
+    return aq, bq, sa, sb
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (512, 512, 512), (1024, 1024, 1024), (32, 1024, 2048), (100, 300, 640),
+                                   (8, 128, 256), (2048, 1024, 512)])
+@pytest.mark.parametrize("streamk", [False, True])
+def test_a8w8(m, n, k, streamk):
+    import tritonblas_amd as tb
+    _say(f"a8w8 {m}x{n}x{k} streamk={streamk}")
+    aq, bq, sa, sb = _a8w8_case(m, n, k)
+    a = aq.cuda()
+    b = bq.T.contiguous().cuda().T            # (K, N) view, K-contiguous like a stored (N, K) weight
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, c.dtype, a.device, streamk=streamk)
+    cfg = tb.matmul_preamble(sel)
+    tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, cfg, enable_streamk=streamk)
+    _check(c.cpu(), OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q)
+    assert cfg.status() == 0
+
+
+@pytest.mark.parametrize("tile", [(256, 256, 128), (128, 128, 128), (64, 64, 128), (32, 128, 256)])
+def test_every_fp8_tile_variant(tile):
+    import tritonblas_amd as tb
+    m, n, k = 384, 640, 1024
+    aq, bq, sa, sb = _a8w8_case(m, n, k, seed=7)
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb)
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.bfloat16, a.device)
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = tile
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, None)
+    _check(c.cpu(), want, torch.bfloat16, TOL_Q)
+
+
+@pytest.mark.parametrize("transA,transB", [("T", "T"), ("N", "N"), ("N", "T")])
+def test_a8w8_other_layouts_take_the_gather_kernel(transA, transB):
+    import tritonblas_amd as tb
+    m, n, k = 192, 160, 320
+    aq, bq, sa, sb = _a8w8_case(m, n, k, seed=9)
+    a, b = _layout(aq.view(torch.uint8), transA).view(torch.float8_e4m3fn), _layout(bq.contiguous().view(torch.uint8), transB).view(torch.float8_e4m3fn)
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    tb.matmul_a8w8(a, b, sa.cuda(), sb.cuda(), c)
+    _check(c.cpu(), OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q)
+
+
+# ---- schedules ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k", [(768, 1024, 512), (512, 1024, 768), (2048, 1024, 512), (16, 16, 4096), (300, 200, 192)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_work_stealing_is_bit_identical_to_static(m, n, k, dtype):
+    import tritonblas_amd as tb
+    _say(f"work stealing {m}x{n}x{k} {dtype}")
+    a, b = _rand((m, k), dtype, 11, 0.5).cuda(), _rand((k, n), dtype, 12, 0.5).cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device)
+    cfg = tb.matmul_preamble(sel)
+    c0 = torch.zeros(m, n, dtype=dtype, device="cuda")
+    tb.matmul_lt(a, b, c0, sel, cfg)
+    for rep in range(3):   # the queues rearm themselves: no reset between launches
+        c1 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        tb.matmul_lt(a, b, c1, sel, cfg, work_stealing=True)
+        assert torch.equal(c0, c1), f"launch {rep}"
+
+
+@pytest.mark.parametrize("m,n,k,grid", [(256, 256, 4096, 64), (128, 128, 8192, 256), (768, 1024, 512, 100), (300, 200, 1920, 37),
+                                       (32, 512, 8192, 256), (64, 64, 64, 8)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_streamk_explicit_grid(m, n, k, grid, dtype):
+    import tritonblas_amd as tb
+    _say(f"stream-k {m}x{n}x{k} grid={grid} {dtype}")
+    a_cpu, b_cpu = _rand((m, k), dtype, 13, 0.5), _rand((k, n), dtype, 14, 0.5)
+    want = OG.ref_gemm(a_cpu, b_cpu, torch.float32)
+    a, b = a_cpu.cuda(), b_cpu.cuda()
+    for rep in range(2):   # the flags carry an epoch: a second launch needs no reset
+        c = tb.matmul(a, b, enable_streamk=True, sk_grid=grid)
+        _check(c.cpu(), want, dtype, TOL_16)
+
+
+def test_streamk_decode_shape_small():
+    """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly."""
+    import tritonblas_amd as tb
+    m, n, k = 32, 1024, 7168
+    aq, bq, sa, sb = _a8w8_case(m, n, k, seed=21)
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, c.dtype, a.device, streamk=True)
+    cfg = tb.matmul_preamble(sel)
+    for _ in range(2):
+        tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, cfg, enable_streamk=True)
+    _check(c.cpu(), OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q)
+    assert cfg.status() == 0
+
+
+# ---- MXFP4 --------------------------------------------------------------------------------------
+def _fp4_case(m, n, k, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.standard_normal((n, k)).astype(np.float32)
+    xq, xs = OM.mxfp4_quant(x)
+    wq, ws = OM.mxfp4_quant(w)
+    return (torch.from_numpy(t) for t in (xq, wq, xs, ws))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (256, 256, 256), (512, 512, 512), (1024, 1024, 1024), (100, 72, 640),
+                                   (2048, 2048, 2048), (32, 256, 1024), (128, 128, 96)])
+def test_matmul_fp4(m, n, k):
+    import tritonblas_amd as tb
+    _say(f"fp4 {m}x{n}x{k}")
+    xq, wq, xs, ws = _fp4_case(m, n, k, 5)
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda())
+    _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.bfloat16, TOL_Q)
+
+
+@pytest.mark.parametrize("tile", [(256, 256, 256), (128, 128, 256), (128, 128, 128), (64, 64, 256)])
+def test_every_fp4_tile_variant(tile):
+    import tritonblas_amd as tb
+    m, n, k = 320, 448, 1024
+    xq, wq, xs, ws = _fp4_case(m, n, k, 6)
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda(), block_m=tile[0], block_n=tile[1], block_k=tile[2])
+    _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.bfloat16, TOL_Q)
+
+
+def test_fp4_scale_extremes():
+    """Scale bytes far from 127 and per-block varying scales must be honoured exactly."""
+    import tritonblas_amd as tb
+    m, n, k = 64, 64, 256
+    rng = np.random.default_rng(8)
+    xq = torch.from_numpy(rng.integers(0, 256, (m, k // 2), dtype=np.uint8))
+    wq = torch.from_numpy(rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
+    xs = torch.from_numpy(rng.integers(100, 150, (m, k // 32), dtype=np.uint8))
+    ws = torch.from_numpy(rng.integers(100, 150, (n, k // 32), dtype=np.uint8))
+    c = torch.zeros(m, n, dtype=torch.float32, device="cuda")
+    tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda())
+    _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.float32, 1e-5)
+
+
+# ---- grouped MoE --------------------------------------------------------------------------------
+@pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [0, 0, 5]])
+def test_grouped_a8w8(counts):
+    import tritonblas_amd as tb
+    _say(f"grouped counts={counts}")
+    E, n, k = len(counts), 384, 512
+    m = sum(counts)
+    offsets = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(4)).bfloat16()
+    w = torch.randn(E, n, k, generator=torch.Generator().manual_seed(10004)).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    wq, sw = OG.quantize_per_channel_fp8(w, axis=2)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda())
+    want = OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True)
+    _check(c.cpu(), want, torch.bfloat16, TOL_Q)
+    # permuting experts permutes the row blocks
+    if E > 1:
+        perm = list(reversed(range(E)))
+        rows = torch.cat([torch.arange(int(offsets[e]), int(offsets[e + 1])) for e in perm])
+        off2 = torch.tensor([0] + list(np.cumsum([counts[e] for e in perm])), dtype=torch.int32)
+        c2 = torch.empty_like(c)
+        tb.grouped_matmul_a8w8(aq[rows].cuda(), wq[perm].cuda(), sa[rows].cuda(), sw[perm].cuda(), c2, off2.cuda())
+        assert torch.equal(c2.cpu(), c.cpu()[rows])

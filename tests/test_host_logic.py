@@ -1,0 +1,148 @@
+"""Host-side logic that needs no GPU: the LDS model and Stream-K grid model restated from the
+reference, the shared library's exports, the analytical selector, and argument validation."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import selector as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# --- LDS model: the reference's known answers (tests/test_lds_estimation.py:44-150) --------------
+@pytest.mark.parametrize("args,want", [
+    ((128, 128, 64, 2, 2, 1), 128 * 64 * 2), ((256, 64, 64, 2, 2, 1), 256 * 64 * 2), ((64, 256, 64, 2, 2, 1), 64 * 256 * 2),
+    ((128, 128, 64, 2, 2, 2), 32768), ((256, 256, 64, 2, 2, 2), 65536), ((128, 128, 64, 2, 2, 3), 65536),
+    ((128, 64, 64, 2, 2, 2), 24576), ((256, 128, 64, 2, 2, 2), 49152), ((64, 64, 32, 2, 2, 2), 8192),
+    ((128, 256, 64, 2, 2, 2), 49152), ((64, 64, 32, 4, 4, 2), 16384), ((128, 128, 32, 4, 4, 2), 32768),
+    ((128, 128, 64, 4, 4, 2), 65536), ((128, 128, 64, 1, 2, 2), 24576), ((128, 128, 64, 0.5, 0.5, 2), 8192),
+])
+def test_lds_known_answers(args, want):
+    from tritonblas_amd.origami import estimate_triton_lds_bytes
+    assert O.estimate_lds_bytes(*args) == want
+    assert estimate_triton_lds_bytes(*args) == want
+
+
+def test_lds_capacity_known_answers():
+    from tritonblas_amd.origami import check_triton_lds_capacity
+    for fn in (O.check_lds_capacity, check_triton_lds_capacity):
+        assert fn(64, 64, 32, 2, 2, 65536, 2) is True
+        assert fn(256, 256, 64, 4, 4, 65536, 2) is False
+        assert fn(256, 256, 64, 2, 2, 65536, 2) is True
+        assert fn(128, 128, 64, 2, 2, 65536, 3) is True
+        assert fn(128, 128, 64, 2, 2, 65536, 4) is False
+        assert fn(128, 128, 64, 0.5, 0.5, 0, 2) is False
+
+
+def test_reference_sk_grid_model_hand_checked():
+    # 8192^2 output with 256^2 tiles on 256 CUs: 1024 tiles, first fraction gives 256, 1024 % 256 == 0
+    assert O.compute_sk_grid(8192, 8192, 8192, 256, 256, 64, 256) == 256
+    # decode shape with a 256-wide tile: 32 tiles < 256 CUs, k split by 8 -> 256 (divides? 32 % 256 != 0 -> tiles)
+    assert O.compute_sk_grid(32, 8192, 28672, 256, 256, 128, 256) == 32
+    # a non-divisor candidate falls back to the tile count
+    assert O.compute_sk_grid(4864, 8192, 4160, 256, 256, 64, 256) == 19 * 32
+    # 608 tiles on 304 CUs: the first fraction gives 304, which divides the tile count
+    assert O.compute_sk_grid(4864, 8192, 4160, 256, 256, 64, 304) == 304
+    # gfx942-only override: 1024 tiles on 304 CUs leave a last wave of 112 (< 128) -> 256
+    assert O.compute_sk_grid(8192, 8192, 8192, 256, 256, 64, 304) == 256
+    assert [O.ws_counters_per_xcd(t) for t in (1, 512, 513, 1536, 1537, 2048, 2049)] == [8, 8, 4, 4, 2, 2, 1]
+
+
+# --- shared library ------------------------------------------------------------------------------
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "tritonblas_amd.h")).read()
+    return sorted(set(re.findall(r"\b(tb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    syms = _header_symbols()
+    assert set(syms) == set(_lib.EXPORTED_SYMBOLS)
+    for s in syms:
+        assert hasattr(lib, s), s
+    assert lib.tb_abi_version() == 1
+    assert _lib.status_string(0) == "ok" and _lib.status_string(-2) == "Incompatible Dimensions"
+
+
+def test_struct_sizes_match_the_header():
+    """ctypes mirrors vs the C compiler's layout (compiled here with gcc)."""
+    import subprocess
+    import tempfile
+    from tritonblas_amd import _lib
+    src = '#include <stdio.h>\n#include "tritonblas_amd.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu\\n",' \
+          'sizeof(tb_hw),sizeof(tb_problem),sizeof(tb_selection),sizeof(tb_gemm_desc),sizeof(tb_gemm_fp4_desc),' \
+          'sizeof(tb_grouped_gemm_desc),sizeof(tb_quant_desc));return 0;}'
+    with tempfile.TemporaryDirectory() as td:
+        open(os.path.join(td, "s.c"), "w").write(src)
+        subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), "-o", os.path.join(td, "s"), os.path.join(td, "s.c")])
+        sizes = [int(v) for v in subprocess.check_output([os.path.join(td, "s")]).split()]
+    mine = [C.sizeof(t) for t in (_lib.tb_hw, _lib.tb_problem, _lib.tb_selection, _lib.tb_gemm_desc, _lib.tb_gemm_fp4_desc,
+                                  _lib.tb_grouped_gemm_desc, _lib.tb_quant_desc)]
+    assert mine == sizes
+
+
+def test_default_hardware_is_mi355x():
+    from tritonblas_amd import _lib
+    hw = _lib.tb_hw()
+    assert _lib.load().tb_device_info(-1, hw) == 0
+    assert (hw.n_cu, hw.num_xcd, hw.cu_per_xcd, hw.lds_bytes, hw.arch) == (256, 8, 32, 163840, b"gfx950")
+
+
+def test_selector_properties_and_lds_fit():
+    """Mirror of the reference's only selector pin (tests/test_lds_estimation.py:211-228): the chosen
+    tile fits the LDS of the part; plus the attribute surface the launchers read."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    for shape, dt, bits in [((8192, 28672, 8192), torch.float8_e4m3fn, 8), ((8192, 8192, 8192), torch.bfloat16, 16),
+                            ((1024, 1024, 1024), torch.float16, 16), ((8192, 8192, 16384), "f4", 4), ((15, 17, 512), torch.bfloat16, 16)]:
+        for sk in (False, True):
+            s = tb.OrigamiMatmulSelector(*shape, dt, dt, torch.bfloat16, torch.device("cuda"), streamk=sk)
+            assert s._hardware.N_CU == 256 and s._hardware.NUM_XCD == 8 and s._hardware.lds_capacity == 163840
+            assert s._hardware.arch.name == "gfx950" and s._N_CU == 256 and s._ACTIVE_CU == 256
+            assert s._sel.lds_bytes <= s._hardware.lds_capacity
+            n = _lib.load().tb_list_tiles(_lib.tb_dtype(dt), None, 0)
+            buf = (C.c_int32 * (3 * n))()
+            _lib.load().tb_list_tiles(_lib.tb_dtype(dt), buf, n)
+            tiles = {(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)}
+            assert (s.block_m, s.block_n, s.block_k) in tiles
+            assert s.group_m == min(8, -(-shape[0] // s.block_m)) and s.num_sms == 8
+            assert s.even_k == (shape[2] % s.block_k == 0)
+            assert s.sk_grid >= 1 and s.num_stages >= 2 and s.waves_per_eu >= 1
+            total = -(-shape[0] // s.block_m) * -(-shape[1] // s.block_n)
+            assert s.COUNTERS_PER_XCD == O.ws_counters_per_xcd(total)
+
+
+def test_argument_validation_without_a_gpu():
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    assert lib.tb_gemm(None, None) == _lib.TB_ERR_NULL_POINTER
+    d = _lib.tb_gemm_desc()
+    assert lib.tb_gemm(d, None) == _lib.TB_ERR_BAD_ARGUMENT          # struct_bytes not set
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+    d.a_type, d.b_type = _lib.TB_F16, _lib.TB_BF16
+    assert lib.tb_gemm(d, None) == _lib.TB_ERR_BAD_DTYPE
+    d.b_type = _lib.TB_F16
+    assert lib.tb_gemm(d, None) == _lib.TB_ERR_NULL_POINTER
+    q = _lib.tb_quant_desc()
+    q.struct_bytes = C.sizeof(_lib.tb_quant_desc)
+    assert lib.tb_hadamard_mxfp4_quant(q, None) == _lib.TB_ERR_NULL_POINTER
+    assert lib.tb_select(None, None, None) == _lib.TB_ERR_NULL_POINTER
+    with pytest.raises(AssertionError, match="Incompatible Dimensions"):
+        _lib.check(_lib.TB_ERR_BAD_SHAPE)
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.TB_ERR_BAD_TILE)
+
+
+def test_python_api_refuses_cpu_tensors():
+    import tritonblas_amd as tb
+    a = torch.zeros(16, 16, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="Incompatible Dimensions"):
+        tb.matmul_lt(a, torch.zeros(8, 16, dtype=torch.float16), a, None, None)
+    with pytest.raises(RuntimeError, match="GPU"):
+        tb.matmul_lt(a, a, a.clone(), None, None)
+    with pytest.raises(RuntimeError, match="differentiation"):
+        tb.matmul(a.requires_grad_(), a, out=torch.zeros(16, 16, dtype=torch.float16))

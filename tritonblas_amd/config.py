@@ -1,0 +1,103 @@
+"""Launch state kept between calls: one device workspace that holds the work-stealing queue
+counters or the Stream-K flags + partial tiles (reference include/tritonblas/config.py:10-134).
+
+Layout of the workspace (bytes): [0, 256) control words (status, done counter); then either
+``num_xcd * counters_per_xcd`` queue counters, one per 256-byte line (work stealing), or ``grid``
+32-bit flags followed by ``grid`` fp32 partial tiles (Stream-K).  Stream-K flags carry the launch
+epoch, so nothing has to be cleared between launches; the work-stealing queues are rearmed by the
+kernel itself.  ``reset()`` is still available after an aborted launch.
+"""
+import torch
+
+from . import _lib
+
+COUNTER_STRIDE = 64   # int32 between counters = 256 bytes
+MAX_SK_TILES = 512
+_CTL_BYTES = 256
+
+
+class MatmulConfig:
+    def __init__(self, device: torch.device, workspace: torch.Tensor, selector=None, mask: torch.Tensor = None,
+                 global_atomic: bool = False):
+        self.device = device
+        self.workspace = workspace
+        self.selector = selector
+        self.mask = mask
+        self.global_atomic = global_atomic
+        self.epoch = 0
+
+    def ensure(self, nbytes: int):
+        """Grow the workspace to at least nbytes (zero-initialised)."""
+        if self.workspace is None or self.workspace.numel() < nbytes:
+            self.workspace = torch.zeros(int(nbytes), dtype=torch.uint8, device=self.device)
+            self.epoch = 0
+        return self.workspace
+
+    def next_epoch(self) -> int:
+        self.epoch = (self.epoch % 0x7FFFFFFF) + 1
+        return self.epoch
+
+    # views under the reference's attribute names -------------------------------------------------
+    @property
+    def tile_counter(self):
+        return self.workspace[_CTL_BYTES:].view(torch.int32)
+
+    @property
+    def locks(self):
+        grid = self.selector.sk_grid if self.selector is not None else 0
+        return self.workspace[_CTL_BYTES:_CTL_BYTES + 4 * grid].view(torch.int32)
+
+    @property
+    def P(self):
+        sel = self.selector
+        grid = sel.sk_grid
+        off = _CTL_BYTES + ((grid * 4 + 255) // 256) * 256
+        blk = sel.block_m * sel.block_n
+        return self.workspace[off:off + grid * blk * 4].view(torch.float32).view(grid, blk)
+
+    def status(self) -> int:
+        """Control word 0: non-zero after a Stream-K wait ran into its poll bound (synchronises)."""
+        return int(self.workspace[:4].view(torch.int32).item())
+
+    def reset(self, streamk: bool = False, work_stealing: bool = False):
+        """Clear mutable state (reference config.py:54-75)."""
+        if (streamk or work_stealing) and self.workspace is not None:
+            self.workspace.zero_()
+            self.epoch = 0
+
+    def __repr__(self):
+        n = 0 if self.workspace is None else self.workspace.numel()
+        return f"MatmulConfig(device={self.device!r}, workspace_bytes={n}, epoch={self.epoch})"
+
+
+def workspace_bytes_for(selector, m=None, n=None, k=None) -> int:
+    """Bytes that cover both the work-stealing and the Stream-K schedule for the selector's tile."""
+    lib = _lib.load()
+    need = 0
+    for sched, grid in ((_lib.TB_SCHED_WORK_STEALING, 0), (_lib.TB_SCHED_STREAMK, selector.sk_grid if selector.streamk else 0)):
+        d = _lib.tb_gemm_desc()
+        d.struct_bytes = _lib.C.sizeof(_lib.tb_gemm_desc)
+        d.a_type = d.b_type = _lib.tb_dtype(selector._a_dtype)
+        d.c_type = _lib.tb_dtype(selector._out_dtype)
+        d.m, d.n, d.k = selector._m, selector._n, selector._k
+        d.a_stride_m, d.a_stride_k = selector._k, 1
+        d.b_stride_k, d.b_stride_n = 1, selector._k
+        d.c_stride_m, d.c_stride_n = selector._n, 1
+        d.block_m, d.block_n, d.block_k = selector.block_m, selector.block_n, selector.block_k
+        d.schedule, d.grid = sched, grid
+        d.counters_per_xcd = selector.COUNTERS_PER_XCD
+        need = max(need, lib.tb_workspace_bytes(d))
+    return int(need)
+
+
+def matmul_preamble(selector, device: torch.device = None) -> MatmulConfig:
+    """Allocate the launch state for a selector (reference config.py:86-134)."""
+    if device is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    need = max(workspace_bytes_for(selector), _CTL_BYTES)
+    workspace = torch.zeros(need, dtype=torch.uint8, device=device)
+    n_cu, active = selector._N_CU, selector._ACTIVE_CU
+    mask = torch.ones(n_cu, dtype=torch.int32, device=device)
+    if active < n_cu:
+        mask[active:] = 0
+    return MatmulConfig(device=device, workspace=workspace, selector=selector, mask=mask)

@@ -1,0 +1,796 @@
+// Device side of the tile GEMM family for gfx950 (MI355X): LDS-staged operands, 16x16 MFMA tiles,
+// fused scale/bias/cast epilogue, and the four tile schedules (data-parallel, work-stealing queues,
+// Stream-K with partial-tile fixup, grouped expert table).
+//
+// One kernel template covers every element type: operands are moved as 16-byte "chunks" along K,
+// both operands sit K-major in LDS, and only the MFMA instruction and the chunk->lane assignment
+// depend on the type.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+namespace tb {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4 };
+enum : int { MODE_STATIC = 0, MODE_WS = 1, MODE_SK = 2, MODE_GROUPED = 3 };
+enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
+
+// Word offsets inside the control block at the head of a workspace.
+enum : int { CTL_STATUS = 0, CTL_DONE = 1, CTL_WORDS = 64 };
+constexpr int COUNTER_STRIDE = 64;  // ints between queue counters: one 256-byte line each
+
+struct GemmParams {
+  const uint8_t* A;
+  const uint8_t* B;
+  uint8_t* C;
+  const float* sa;
+  const float* sb;
+  const uint8_t* bias;
+  const uint8_t* mxa;
+  const uint8_t* mxb;
+  int32_t M, N;
+  int64_t KU;                    // K extent in storage units (elements; bytes for packed fp4)
+  int64_t a_sr, a_sk;            // strides in storage units: row (m) and k
+  int64_t b_sr, b_sk;            // row (n) and k
+  int64_t c_sm, c_sn;            // elements
+  int64_t mxa_sr, mxa_sk, mxb_sr, mxb_sk;  // bytes
+  int64_t bias_stride;
+  int32_t c_type, bias_type;
+  int32_t a_vec, b_vec, c_vec;   // 16-byte vector access is legal for this operand
+  int32_t mx_vec;                // scale rows can be read KSUB bytes at a time
+  int32_t tiles_m, tiles_n, total_tiles, k_iters;
+  int32_t group_m, num_xcds, chunk;
+  int32_t mode;
+  // Stream-K
+  int32_t sk_tiles;
+  float* P;
+  uint32_t* flags;
+  uint32_t epoch, spin_limit;
+  uint32_t* ctl;
+  // work stealing
+  int32_t* counters;
+  int32_t counters_per_xcd;
+  const int32_t* cu_mask;
+  // grouped
+  const int32_t* group_offsets;
+  int32_t num_groups;
+  int64_t b_group_stride;   // storage units between consecutive experts' weights
+  int64_t sb_group_stride;  // floats
+};
+
+struct TileCtx {
+  int m0, n0, m_lim, n_lim;
+  const uint8_t* B;
+  const float* sb;
+};
+
+template <int DT_, int BM_, int BN_, int BKB_, int WM_, int WN_, int ALAY_, int BLAY_, int MINB_ = 1,
+          bool FAST_ = true, int STAGES_ = 2>
+struct Tile {
+  static constexpr int DT = DT_, BM = BM_, BN = BN_, BKB = BKB_, WM = WM_, WN = WN_;
+  static constexpr int ALAY = ALAY_, BLAY = BLAY_, MINB = MINB_, STAGES = STAGES_;
+  // FAST: operands are 16-byte aligned, unit stride along their contiguous index, K is a multiple
+  // of the K step (and row counts of M-contiguous operands multiples of 8): loaders carry no
+  // bounds handling besides clamping rows.  !FAST: element-wise gathers, any strides, any K.
+  static constexpr bool FAST = FAST_;
+  static constexpr bool DMA = FAST && ALAY == LAY_K && BLAY == LAY_K;  // global -> LDS without registers
+  static constexpr int THREADS = WM * WN * 64;
+  static constexpr int USZ = (DT == DT_F16 || DT == DT_BF16) ? 2 : 1;  // bytes per storage unit
+  static constexpr int UPC = 16 / USZ;                                 // units per 16-byte chunk
+  static constexpr int CPR = BKB / 16;                                 // chunks per tile row
+  static constexpr int UPS = CPR * UPC;                                // units per K step
+  static constexpr int EPU = (DT == DT_FP4) ? 2 : 1;                   // elements per unit
+  static constexpr int BK = UPS * EPU;                                 // elements per K step
+  static constexpr int KS = (DT == DT_FP8) ? 8 : 4;                    // chunks one MFMA consumes per row
+  static constexpr int KSUB = CPR / KS;                                // MFMA k-slices per K step
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int TM = WTM / 16, TN = WTN / 16;
+  static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  // XOR swizzle of the chunk index so that 16 rows read at one k hit 16 different bank groups.
+  static constexpr int RPL = (CPR >= 16) ? 1 : 16 / CPR;   // tile rows per 256-byte LDS line
+  static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // swizzle period
+  static_assert(CPR % KS == 0, "K step must hold whole MFMA slices");
+  static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be MFMA aligned");
+  static_assert(DT != DT_FP4 || KSUB == 1 || KSUB == 2 || KSUB == 4, "fp4 scale packing");
+  static_assert(STAGES == 2 || (DMA && STAGES == 3), "deeper pipelines need the LDS-direct loader");
+  static_assert((BM * CPR) % 64 == 0 && (BN * CPR) % 64 == 0, "whole waves per operand copy");
+  __device__ static __forceinline__ int swz(int row) { return (row / RPL) % SWM; }
+};
+
+struct LaneInfo {
+  int tid, lane, r, g, wm0, wn0;
+};
+
+// ------------------------------------------------------------------------------------------------
+// integer tile-order functions (same arithmetic as the host-side schedule tests check)
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int chiplet_transform_chunked(int pid, int num_wg, int num_xcds, int chunk) {
+  int block = num_xcds * chunk;
+  if (pid > (num_wg / block) * block) return pid;
+  int local = pid / num_xcds;
+  int chunk_idx = local / chunk, pos = local % chunk, xcd = pid % num_xcds;
+  return chunk_idx * block + xcd * chunk + pos;
+}
+
+__device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int group_m, int& pm, int& pn) {
+  int in_group = group_m * tiles_n;
+  int gid = tile / in_group;
+  int first = gid * group_m;
+  int gsz = min(tiles_m - first, group_m);
+  int rem = tile % in_group;
+  pm = first + rem % gsz;
+  pn = rem / gsz;
+}
+
+// ------------------------------------------------------------------------------------------------
+// global -> LDS operand movement
+// ------------------------------------------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ v4i gather_units(const uint8_t* rowp, int64_t ku, int64_t s_k, int64_t KU) {
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if constexpr (T::USZ == 2) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      int64_t k = ku + u;
+      uint32_t v = (k < KU) ? (uint32_t)(*(const uint16_t*)(rowp + k * s_k * 2)) : 0u;
+      w[u >> 1] |= v << (16 * (u & 1));
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      int64_t k = ku + u;
+      uint32_t v = (k < KU) ? (uint32_t)rowp[k * s_k] : 0u;
+      w[u >> 2] |= v << (8 * (u & 3));
+    }
+  }
+  v4i out = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  return out;
+}
+
+// LDS image of an operand tile: ROWS rows of CPR chunks; chunk c of row r sits at chunk slot
+// r*CPR + (c ^ swz(r)).  Slot q is filled by thread q % THREADS in round q / THREADS, so a wave
+// always fills 64 consecutive slots (what the LDS-direct load requires).
+template <class T, int ROWS, int LAY>
+struct Operand {
+  static constexpr int CHUNKS = ROWS * T::CPR;
+  static constexpr int NCH = (CHUNKS + T::THREADS - 1) / T::THREADS;  // slots per thread
+  static constexpr int RG = ROWS / 8;                                  // 8-row groups (LAY_M)
+  static constexpr int NBLK = RG * T::CPR;                             // 8x8 blocks (LAY_M)
+  static constexpr int NBT = (NBLK + T::THREADS - 1) / T::THREADS;
+  static constexpr bool TRANSPOSING = T::FAST && LAY == LAY_M;
+  static constexpr int NREG = TRANSPOSING ? NBT * 8 : NCH;
+  static constexpr int NOFF = TRANSPOSING ? NBT : NCH;
+  static_assert(!TRANSPOSING || T::USZ == 2, "transposing loader is for 16-bit operands");
+
+  struct St {
+    const uint8_t* base;     // FAST: tile origin; else matrix origin
+    uint32_t off[NOFF];      // FAST: per-slot byte offset from the K-step origin
+    int64_t s_row, s_k;      // storage units
+    int row0, row_lim;
+  };
+
+  __device__ static __forceinline__ void init(St& st, const uint8_t* mat, int64_t s_row, int64_t s_k, int row0,
+                                              int row_lim, int tid) {
+    st.s_row = s_row; st.s_k = s_k; st.row0 = row0; st.row_lim = row_lim;
+    const int rows_valid = row_lim - row0;
+    if constexpr (!T::FAST) {
+      st.base = mat;
+    } else if constexpr (LAY == LAY_K) {
+      st.base = mat + (int64_t)row0 * s_row * T::USZ;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        int q = i * T::THREADS + tid;
+        int row = q / T::CPR, pc = q % T::CPR;
+        int c = pc ^ T::swz(row);
+        int rowc = min(row, rows_valid - 1);
+        st.off[i] = (uint32_t)(rowc * (int)(s_row * T::USZ) + c * 16);
+      }
+    } else {
+      st.base = mat + (int64_t)row0 * 2;
+      const int last = ((rows_valid - 1) / 8) * 8;
+#pragma unroll
+      for (int ib = 0; ib < NBT; ++ib) {
+        int b = ib * T::THREADS + tid;
+        int rg = b % RG, c = b / RG;
+        st.off[ib] = (uint32_t)(min(rg * 8, last) * 2 + c * 8 * (int)(s_k * 2));
+      }
+    }
+  }
+
+  // K-step origin for iteration `it`
+  __device__ static __forceinline__ const uint8_t* step_ptr(const St& st, int it) {
+    if constexpr (!T::FAST) return st.base;
+    else if constexpr (LAY == LAY_K) return st.base + (int64_t)it * T::BKB;
+    else return st.base + (int64_t)it * T::UPS * st.s_k * 2;
+  }
+
+  // LDS-direct copy of K step `it` into `lds` (no registers involved)
+  __device__ static __forceinline__ void dma(const St& st, int it, uint8_t* lds, int tid) {
+    const uint8_t* gp = step_ptr(st, it);
+    const int wave_slot = __builtin_amdgcn_readfirstlane(tid & ~63);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      if (CHUNKS % T::THREADS != 0 && i * T::THREADS + wave_slot >= CHUNKS) continue;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gp + st.off[i]),
+                                       (__attribute__((address_space(3))) void*)(lds + (i * T::THREADS + wave_slot) * 16),
+                                       16, 0, 0);
+    }
+  }
+
+  __device__ static __forceinline__ void gload(v4i (&r)[NREG], const St& st, int it, int64_t KU, int tid) {
+    const uint8_t* gp = step_ptr(st, it);
+    if constexpr (!T::FAST) {
+      const int64_t ku0 = (int64_t)it * T::UPS;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        int q = i * T::THREADS + tid;
+        if (CHUNKS % T::THREADS != 0 && q >= CHUNKS) continue;
+        int row = q / T::CPR, pc = q % T::CPR;
+        int c = pc ^ T::swz(row);
+        int64_t grow = min(st.row0 + row, st.row_lim - 1);
+        r[i] = gather_units<T>(gp + grow * st.s_row * T::USZ, ku0 + (int64_t)c * T::UPC, st.s_k, KU);
+      }
+    } else if constexpr (LAY == LAY_K) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        if (CHUNKS % T::THREADS != 0 && i * T::THREADS + tid >= CHUNKS) continue;
+        r[i] = *(const v4i*)(gp + st.off[i]);
+      }
+    } else {
+      const int64_t ldk = st.s_k * 2;
+#pragma unroll
+      for (int ib = 0; ib < NBT; ++ib) {
+        if (NBLK % T::THREADS != 0 && ib * T::THREADS + tid >= NBLK) continue;
+        uint32_t w[8][4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          v4i v = *(const v4i*)(gp + st.off[ib] + j * ldk);
+          w[j][0] = v.x; w[j][1] = v.y; w[j][2] = v.z; w[j][3] = v.w;
+        }
+        // 8x8 transpose of 16-bit values: out row i, dword d holds k = 2d (low half) and 2d+1 (high).
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          uint32_t o[4];
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            uint32_t lo = w[2 * d][i >> 1], hi = w[2 * d + 1][i >> 1];
+            o[d] = (i & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+          }
+          v4i ov = {(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+          r[ib * 8 + i] = ov;
+        }
+      }
+    }
+  }
+
+  __device__ static __forceinline__ void sstore(uint8_t* lds, const v4i (&r)[NREG], int tid) {
+    if constexpr (!TRANSPOSING) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        int q = i * T::THREADS + tid;
+        if (CHUNKS % T::THREADS != 0 && q >= CHUNKS) continue;
+        *(v4i*)(lds + q * 16) = r[i];
+      }
+    } else {
+#pragma unroll
+      for (int ib = 0; ib < NBT; ++ib) {
+        int b = ib * T::THREADS + tid;
+        if (NBLK % T::THREADS != 0 && b >= NBLK) continue;
+        int rg = b % RG, c = b / RG;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          int row = rg * 8 + i;
+          *(v4i*)(lds + row * T::BKB + ((c ^ T::swz(row)) << 4)) = r[ib * 8 + i];
+        }
+      }
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------------
+// LDS -> MFMA operand fragments
+// ------------------------------------------------------------------------------------------------
+template <class T>
+struct Frag {
+  using type = typename std::conditional<T::DT == DT_FP8, v8i, v4i>::type;
+
+  // row: tile row of this lane (wave row base + 16*t + lane%16); g = lane/16; m = swizzle mask of row.
+  __device__ static __forceinline__ type read(const uint8_t* lds, int row, int ks, int g, int m) {
+    const uint8_t* rp = lds + row * T::BKB;
+    if constexpr (T::DT == DT_FP8) {
+      int c0 = ks * 8 + 2 * g;
+      v4i lo = *(const v4i*)(rp + ((c0 ^ m) << 4));
+      v4i hi = *(const v4i*)(rp + (((c0 + 1) ^ m) << 4));
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    } else if constexpr (T::DT == DT_FP4) {
+      int c = g * T::KSUB + ks;  // lane group g owns KSUB consecutive 32-blocks: their scale bytes are adjacent
+      return *(const v4i*)(rp + ((c ^ m) << 4));
+    } else {
+      int c = ks * 4 + g;
+      return *(const v4i*)(rp + ((c ^ m) << 4));
+    }
+  }
+};
+
+// D(16x16) += X(16xk) * Y(16xk)^T; lane l holds D[4*(l/16)+j][l%16], j = 0..3.
+template <class T, int KSI>
+__device__ __forceinline__ v4f mma(typename Frag<T>::type x, typename Frag<T>::type y, v4f c, uint32_t sx, uint32_t sy) {
+  if constexpr (T::DT == DT_F16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, x), __builtin_bit_cast(h8, y), c, 0, 0, 0);
+  } else if constexpr (T::DT == DT_BF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, x), __builtin_bit_cast(bf8, y), c, 0, 0, 0);
+  } else if constexpr (T::DT == DT_FP8) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
+  } else {
+    v8i x8 = {x.x, x.y, x.z, x.w, 0, 0, 0, 0};
+    v8i y8 = {y.x, y.y, y.z, y.w, 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x8, y8, c, 4, 4, KSI, sx, KSI, sy);
+  }
+}
+
+// E8M0 scale bytes of one lane for one K step: KSUB consecutive 32-blocks starting at kb, packed
+// little-endian into a dword; blocks at or past kb_total read as 127 (= 1.0) so that zero-filled
+// data cannot meet a NaN scale.
+template <class T>
+__device__ __forceinline__ uint32_t load_mx(const uint8_t* rowp, int64_t s_k, int64_t kb, int64_t kb_total, bool vec) {
+  if (vec && kb + T::KSUB <= kb_total) {
+    if constexpr (T::KSUB == 4) return *(const uint32_t*)(rowp + kb);
+    if constexpr (T::KSUB == 2) return *(const uint16_t*)(rowp + kb);
+    if constexpr (T::KSUB == 1) return *(rowp + kb);
+  }
+  uint32_t w = 0;
+#pragma unroll
+  for (int j = 0; j < T::KSUB; ++j) {
+    uint32_t v = (kb + j < kb_total) ? (uint32_t)rowp[(kb + j) * s_k] : 127u;
+    w |= v << (8 * j);
+  }
+  return w;
+}
+
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0) only
+
+// ------------------------------------------------------------------------------------------------
+// K loop: accumulates k iterations [it0, it1) of one output tile
+// ------------------------------------------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc, int it0, int it1,
+                                         v4f (&acc)[T::TM][T::TN], uint8_t* lds, const LaneInfo& li) {
+  using OA = Operand<T, T::BM, T::ALAY>;
+  using OB = Operand<T, T::BN, T::BLAY>;
+  using frag_t = typename Frag<T>::type;
+  typename OA::St sa;
+  typename OB::St sb;
+  OA::init(sa, p.A, p.a_sr, p.a_sk, tc.m0, tc.m_lim, li.tid);
+  OB::init(sb, tc.B, p.b_sr, p.b_sk, tc.n0, tc.n_lim, li.tid);
+  uint32_t sca[T::TM], scb[T::TN], nsca[T::TM], nscb[T::TN];
+  const int swm = T::swz(li.r);
+  const int64_t kb_total = (p.KU * T::EPU) / 32;
+
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i] = 0;
+#pragma unroll
+  for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j] = 0;
+
+  auto load_scales = [&](int it, uint32_t(&xa)[T::TM], uint32_t(&xb)[T::TN]) {
+    if constexpr (T::DT == DT_FP4) {
+      int64_t kb = (int64_t)it * T::CPR + li.g * T::KSUB;
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) {
+        int64_t row = min(tc.m0 + li.wm0 + i * 16 + li.r, tc.m_lim - 1);
+        xa[i] = load_mx<T>(p.mxa + row * p.mxa_sr, p.mxa_sk, kb, kb_total, p.mx_vec);
+      }
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+        int64_t row = min(tc.n0 + li.wn0 + j * 16 + li.r, tc.n_lim - 1);
+        xb[j] = load_mx<T>(p.mxb + row * p.mxb_sr, p.mxb_sk, kb, kb_total, p.mx_vec);
+      }
+    }
+  };
+
+  auto compute = [&](const uint8_t* sA, const uint8_t* sB) {
+#pragma unroll
+    for (int ks = 0; ks < T::KSUB; ++ks) {
+      frag_t bf[T::TN];
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) bf[j] = Frag<T>::read(sB, li.wn0 + j * 16 + li.r, ks, li.g, swm);
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) {
+        frag_t af = Frag<T>::read(sA, li.wm0 + i * 16 + li.r, ks, li.g, swm);
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+          // output rows follow the first MFMA operand: feed B there so that one lane owns four
+          // consecutive n of one m (contiguous in a row-major C).
+          if (ks == 0) acc[i][j] = mma<T, 0>(bf[j], af, acc[i][j], scb[j], sca[i]);
+          if (ks == 1) acc[i][j] = mma<T, 1>(bf[j], af, acc[i][j], scb[j], sca[i]);
+          if (ks == 2) acc[i][j] = mma<T, 2>(bf[j], af, acc[i][j], scb[j], sca[i]);
+          if (ks == 3) acc[i][j] = mma<T, 3>(bf[j], af, acc[i][j], scb[j], sca[i]);
+        }
+      }
+    }
+  };
+
+  if constexpr (T::DMA) {
+    constexpr int S = T::STAGES;
+    // stage s of iteration it: lds + ((it - it0) % S) * STAGE_BYTES; copies run S-1 iterations ahead.
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) {
+      if (it0 + s < it1) {
+        OA::dma(sa, it0 + s, lds + s * T::STAGE_BYTES, li.tid);
+        OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
+      }
+    }
+    load_scales(it0, sca, scb);
+    if (S == 3 && it0 + 1 < it1) __builtin_amdgcn_s_waitcnt(0x0F70 | 0);  // conservative: everything landed
+    else wait_vm0();
+    __syncthreads();
+    int stage = 0;
+    for (int it = it0; it < it1; ++it) {
+      const int nxt = it + S - 1;
+      int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
+      if (nxt < it1) {
+        OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
+        OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
+      }
+      if (it + 1 < it1) load_scales(it + 1, nsca, nscb);
+      compute(lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      if (it + 1 < it1) {
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j];
+      }
+      // the next iteration's stage must have landed; with three stages one copy group may stay in flight
+      if (S == 3 && T::DT != DT_FP4 && nxt < it1) {
+        constexpr int NI = OA::NCH + OB::NCH;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (NI & 0xF) | ((NI >> 4) << 14));
+      } else {
+        wait_vm0();
+      }
+      __syncthreads();
+      stage = (stage + 1 == S) ? 0 : stage + 1;
+    }
+  } else {
+    v4i ra[OA::NREG], rb[OB::NREG];
+    uint8_t* sA0 = lds;
+    uint8_t* sB0 = lds + T::A_BYTES;
+    OA::gload(ra, sa, it0, p.KU, li.tid);
+    OB::gload(rb, sb, it0, p.KU, li.tid);
+    load_scales(it0, sca, scb);
+    OA::sstore(sA0, ra, li.tid);
+    OB::sstore(sB0, rb, li.tid);
+    __syncthreads();
+    for (int it = it0; it < it1; ++it) {
+      const int cur = (it - it0) & 1;
+      const bool has_next = it + 1 < it1;
+      if (has_next) {
+        OA::gload(ra, sa, it + 1, p.KU, li.tid);
+        OB::gload(rb, sb, it + 1, p.KU, li.tid);
+        load_scales(it + 1, nsca, nscb);
+      }
+      compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
+      if (has_next) {
+        OA::sstore(sA0 + (cur ^ 1) * T::STAGE_BYTES, ra, li.tid);
+        OB::sstore(sB0 + (cur ^ 1) * T::STAGE_BYTES, rb, li.tid);
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j];
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// epilogue: acc * (sa*sb) + bias -> cast -> store.  Lane holds C[m][n..n+3].
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float load_as_f32(const uint8_t* p, int type) {
+  if (type == DT_F32) return *(const float*)p;
+  if (type == DT_F16) return (float)(*(const _Float16*)p);
+  uint32_t u = (uint32_t)(*(const uint16_t*)p) << 16;
+  return __builtin_bit_cast(float, u);
+}
+
+template <int CT>
+__device__ __forceinline__ void store4(uint8_t* C, int64_t off_el, int64_t sn, v4f v, int nvalid, bool vec) {
+  if constexpr (CT == DT_F32) {
+    float* cp = (float*)C + off_el;
+    if (vec && nvalid >= 4) { *(v4f*)cp = v; return; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (j < nvalid) cp[j * sn] = v[j];
+  } else {
+    uint16_t h[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (CT == DT_F16) h[j] = __builtin_bit_cast(uint16_t, (_Float16)v[j]);
+      else h[j] = __builtin_bit_cast(uint16_t, (__bf16)v[j]);
+    }
+    uint16_t* cp = (uint16_t*)C + off_el;
+    if (vec && nvalid >= 4) {
+      uint2 pk = {(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+      *(uint2*)cp = pk;
+      return;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (j < nvalid) cp[j * sn] = h[j];
+  }
+}
+
+template <class T, int CT>
+__device__ __forceinline__ void epilogue_t(const GemmParams& p, const TileCtx& tc, v4f (&acc)[T::TM][T::TN],
+                                           const LaneInfo& li) {
+  float sav[T::TM];
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i) {
+    int m = tc.m0 + li.wm0 + i * 16 + li.r;
+    sav[i] = (p.sa && m < tc.m_lim) ? p.sa[m] : 1.f;
+  }
+#pragma unroll
+  for (int j = 0; j < T::TN; ++j) {
+    int n = tc.n0 + li.wn0 + j * 16 + 4 * li.g;
+    int nvalid = tc.n_lim - n;
+    v4f sbv = {1.f, 1.f, 1.f, 1.f}, bv = {0.f, 0.f, 0.f, 0.f};
+    if (tc.sb) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) if (q < nvalid) sbv[q] = tc.sb[n + q];
+    }
+    if (p.bias) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (q < nvalid) bv[q] = load_as_f32(p.bias + (int64_t)(n + q) * p.bias_stride * (p.bias_type == DT_F32 ? 4 : 2), p.bias_type);
+    }
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i) {
+      int m = tc.m0 + li.wm0 + i * 16 + li.r;
+      if (m >= tc.m_lim || nvalid <= 0) continue;
+      v4f v = acc[i][j];
+      if (p.sa) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = v[q] * (sav[i] * sbv[q]);
+      }
+      if (p.bias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = v[q] + bv[q];
+      }
+      store4<CT>(p.C, (int64_t)m * p.c_sm + (int64_t)n * p.c_sn, p.c_sn, v, nvalid, p.c_vec);
+    }
+  }
+}
+
+template <class T>
+__device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc, v4f (&acc)[T::TM][T::TN],
+                                         const LaneInfo& li) {
+  if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);
+  else if (p.c_type == DT_F16) epilogue_t<T, DT_F16>(p, tc, acc, li);
+  else epilogue_t<T, DT_F32>(p, tc, acc, li);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stream-K partial tiles: fragment-ordered fp32 in P[slot], one float4 per lane per MFMA tile
+// ------------------------------------------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ void partial_store(float* slot, v4f (&acc)[T::TM][T::TN], int tid) {
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) *(v4f*)(slot + ((size_t)((i * T::TN + j) * T::THREADS + tid) << 2)) = acc[i][j];
+}
+
+template <class T>
+__device__ __forceinline__ void partial_add(const float* slot, v4f (&acc)[T::TM][T::TN], int tid) {
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+      v4f v = *(const v4f*)(slot + ((size_t)((i * T::TN + j) * T::THREADS + tid) << 2));
+      acc[i][j] += v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// work items: which (tile, k range) a workgroup runs next, for each schedule
+// ------------------------------------------------------------------------------------------------
+enum : int { WK_FULL = 0, WK_SK_PUBLISH = 1, WK_SK_OWNER = 2 };
+
+struct Work {
+  TileCtx tc;
+  int it0, it1, kind;
+  int64_t seg_end, tile_end;  // Stream-K owner: global iteration where its segment / its tile ends
+};
+
+__device__ __forceinline__ void plain_tile(const GemmParams& p, int tile, int BM, int BN, TileCtx& tc) {
+  int pm, pn;
+  tile_coords(tile, p.tiles_m, p.tiles_n, p.group_m, pm, pn);
+  tc.m0 = pm * BM; tc.n0 = pn * BN; tc.m_lim = p.M; tc.n_lim = p.N;
+  tc.B = p.B; tc.sb = p.sb;
+}
+
+// Grouped table: experts in order, expert e owns cdiv(rows_e, BM) * tiles_n tiles, m-block fastest.
+__device__ __forceinline__ bool grouped_tile(const GemmParams& p, int tile, int BM, int BN, int USZ, TileCtx& tc) {
+  int acc = 0;
+  for (int e = 0; e < p.num_groups; ++e) {
+    int lo = p.group_offsets[e], hi = p.group_offsets[e + 1];
+    int mb = (hi - lo + BM - 1) / BM;
+    int cnt = mb * p.tiles_n;
+    if (tile < acc + cnt) {
+      int local = tile - acc;
+      tc.m0 = lo + (local % mb) * BM;
+      tc.n0 = (local / mb) * BN;
+      tc.m_lim = hi; tc.n_lim = p.N;
+      tc.B = p.B + (int64_t)e * p.b_group_stride * USZ;
+      tc.sb = p.sb ? p.sb + (int64_t)e * p.sb_group_stride : nullptr;
+      return true;
+    }
+    acc += cnt;
+  }
+  return false;
+}
+
+template <class T>
+struct Sched {
+  int pid, G;
+  int next_tile;          // static / Stream-K data-parallel phase
+  int step;               // work stealing: queue visit index
+  int64_t start, last, q, rem;  // Stream-K iteration range of this workgroup
+  int dp_tiles;
+
+  __device__ __forceinline__ void init(const GemmParams& p) {
+    G = gridDim.x;
+    pid = blockIdx.x;
+    if (p.mode != MODE_WS && p.num_xcds > 1) pid = chiplet_transform_chunked(pid, G, p.num_xcds, p.chunk);
+    next_tile = pid;
+    step = 0;
+    dp_tiles = p.total_tiles - p.sk_tiles;
+    start = last = q = rem = 0;
+    if (p.mode == MODE_SK) {
+      const int64_t total_sk = (int64_t)p.sk_tiles * p.k_iters;
+      q = total_sk / G; rem = total_sk % G;
+      start = (int64_t)dp_tiles * p.k_iters + pid * q + min((int64_t)pid, rem);
+      last = (int64_t)dp_tiles * p.k_iters + (pid + 1) * q + min((int64_t)pid + 1, rem);
+    }
+    if (p.mode == MODE_WS && p.cu_mask && p.cu_mask[pid] == 0) step = 1 << 30;  // masked out: nothing to do
+  }
+
+  __device__ __forceinline__ bool next(const GemmParams& p, Work& w, int* s_bcast, int tid) {
+    w.it0 = 0; w.it1 = p.k_iters; w.kind = WK_FULL; w.seg_end = w.tile_end = 0;
+    if (p.mode == MODE_STATIC) {
+      if (next_tile >= p.total_tiles) return false;
+      plain_tile(p, next_tile, T::BM, T::BN, w.tc);
+      next_tile += G;
+      return true;
+    }
+    if (p.mode == MODE_GROUPED) {
+      if (next_tile < 0) return false;
+      bool ok = grouped_tile(p, next_tile, T::BM, T::BN, T::USZ, w.tc);
+      next_tile = -1;
+      return ok;
+    }
+    if (p.mode == MODE_WS) {
+      // Queues: one counter per (xcd, slot).  A workgroup drains its own queue, then the other
+      // slots of its XCD, then the other XCDs' queues.
+      const int X = p.num_xcds, S = p.counters_per_xcd;
+      const int xcd = pid % X, slot = (pid / X) % S;
+      const int per_xcd = (p.total_tiles + X - 1) / X;
+      while (step < X * S) {
+        int qx = (xcd + step / S) % X;
+        int qs = (slot + step % S) % S;
+        int xbase = qx * per_xcd;
+        int xcnt = max(min(xbase + per_xcd, p.total_tiles) - xbase, 0);
+        int per_slot = (xcnt + S - 1) / S;
+        int sbase = qs * per_slot;
+        int bound = max(min(sbase + per_slot, xcnt) - sbase, 0);
+        if (tid == 0) *s_bcast = (bound > 0) ? atomicAdd(p.counters + (qx * S + qs) * COUNTER_STRIDE, 1) : 0;
+        __syncthreads();
+        int idx = *s_bcast;
+        __syncthreads();
+        if (idx < bound) {
+          plain_tile(p, xbase + sbase + idx, T::BM, T::BN, w.tc);
+          return true;
+        }
+        ++step;
+      }
+      return false;
+    }
+    // MODE_SK: data-parallel tiles first, then this workgroup's share of the Stream-K iterations
+    if (next_tile < dp_tiles) {
+      plain_tile(p, next_tile, T::BM, T::BN, w.tc);
+      next_tile += G;
+      return true;
+    }
+    if (start >= last) return false;
+    const int ipt = p.k_iters;
+    const int tile = (int)(start / ipt);
+    const int64_t tile_first = (int64_t)tile * ipt;
+    const int64_t tile_end = tile_first + ipt;
+    const int64_t end = min(tile_end, last);
+    plain_tile(p, tile, T::BM, T::BN, w.tc);
+    w.it0 = (int)(start - tile_first);
+    w.it1 = (int)(end - tile_first);
+    w.kind = (start != tile_first) ? WK_SK_PUBLISH : WK_SK_OWNER;
+    w.seg_end = end; w.tile_end = tile_end;
+    start = end;
+    return true;
+  }
+};
+
+template <class T>
+__global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmParams p) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_BYTES];
+  __shared__ int s_bcast;
+  LaneInfo li;
+  li.tid = threadIdx.x;
+  li.lane = li.tid & 63;
+  li.r = li.lane & 15;
+  li.g = li.lane >> 4;
+  const int wave = li.tid >> 6;
+  li.wm0 = (wave / T::WN) * T::WTM;
+  li.wn0 = (wave % T::WN) * T::WTN;
+  v4f acc[T::TM][T::TN];
+
+  Sched<T> sched;
+  sched.init(p);
+  Work w;
+  bool failed = false;
+  while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
+    mainloop<T>(p, w.tc, w.it0, w.it1, acc, lds, li);
+    if (w.kind == WK_SK_PUBLISH) {
+      // not the tile's first segment: publish the partial, tagged with this launch's epoch
+      partial_store<T>(p.P + (size_t)sched.pid * (T::BM * T::BN), acc, li.tid);
+      __threadfence();
+      __syncthreads();
+      if (li.tid == 0) __hip_atomic_store(p.flags + sched.pid, p.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      continue;
+    }
+    if (w.kind == WK_SK_OWNER) {
+      // owner of the tile: add the partials of the following workgroups in ascending order
+      int nxt = sched.pid + 1;
+      int64_t cur_end = w.seg_end;
+      while (cur_end < w.tile_end) {
+        if (li.tid == 0) {
+          uint32_t spins = 0;
+          int ok = 1;
+          while (__hip_atomic_load(p.flags + nxt, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
+            if (++spins >= p.spin_limit) { ok = 0; break; }
+            __builtin_amdgcn_s_sleep(2);
+          }
+          s_bcast = ok;
+        }
+        __syncthreads();
+        int ok = s_bcast;
+        __syncthreads();
+        if (!ok) { failed = true; break; }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        partial_add<T>(p.P + (size_t)nxt * (T::BM * T::BN), acc, li.tid);
+        cur_end += sched.q + (nxt < sched.rem ? 1 : 0);
+        ++nxt;
+      }
+      if (failed) break;
+    }
+    epilogue<T>(p, w.tc, acc, li);
+  }
+  if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
+  if (p.mode == MODE_WS && li.tid == 0) {
+    // the last workgroup to leave rearms the queues for the next launch
+    uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
+    if (done == gridDim.x - 1) {
+      for (int qi = 0; qi < p.num_xcds * p.counters_per_xcd; ++qi)
+        __hip_atomic_store(p.counters + qi * COUNTER_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+}  // namespace tb

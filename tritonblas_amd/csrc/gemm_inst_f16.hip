@@ -1,0 +1,21 @@
+// f16 tile GEMM kernels: every tile shape for the four operand layout combinations, plus one
+// element-wise-gather kernel for operands the vector loaders cannot address.
+#include "gemm_variants.h"
+
+namespace tb {
+
+#define TB_LAYOUTS(BM, BN, WM, WN, MINB)                                              \
+  make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_K, LAY_K, MINB, true, 2>>(),      \
+  make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_K, LAY_M, MINB, true, 2>>(),      \
+  make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_M, LAY_K, MINB, true, 2>>(),      \
+  make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_M, LAY_M, MINB, true, 2>>()
+
+const Variant g_variants_f16[] = {
+    TB_LAYOUTS(256, 256, 2, 2, 1),
+    TB_LAYOUTS(128, 128, 2, 2, 2),
+    TB_LAYOUTS(64, 64, 2, 2, 4),
+    make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),
+};
+const int g_num_variants_f16 = sizeof(g_variants_f16) / sizeof(Variant);
+
+}  // namespace tb

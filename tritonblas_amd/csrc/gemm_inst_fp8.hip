@@ -1,0 +1,16 @@
+// FP8 (OCP e4m3) tile GEMM kernels.  The fast kernels take K-major operands; everything else goes
+// through the element-wise-gather kernel.
+#include "gemm_variants.h"
+
+namespace tb {
+
+const Variant g_variants_fp8[] = {
+    make_variant<Tile<DT_FP8, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>>(),
+    make_variant<Tile<DT_FP8, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
+    make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),
+    make_variant<Tile<DT_FP8, 32, 128, 256, 1, 4, LAY_K, LAY_K, 1, true, 3>>(),
+    make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),
+};
+const int g_num_variants_fp8 = sizeof(g_variants_fp8) / sizeof(Variant);
+
+}  // namespace tb

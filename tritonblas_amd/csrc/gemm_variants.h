@@ -1,0 +1,32 @@
+// Host-visible registry of the built GEMM kernel variants.
+#pragma once
+#include <stdint.h>
+#include "gemm_device.h"
+
+namespace tb {
+
+struct Variant {
+  int dt, bm, bn, bk;     // element type and tile in elements
+  int alay, blay;         // operand loaders (LAY_K / LAY_M)
+  int threads, lds_bytes, minb;
+  int fast, stages;       // fast: vector/LDS-direct loaders (alignment + K multiple required)
+  const void* kernel;     // __global__ void (*)(const GemmParams)
+};
+
+template <class T>
+constexpr Variant make_variant() {
+  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::THREADS, T::LDS_BYTES + 16, T::MINB,
+                 T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T>};
+}
+
+// defined one per translation unit
+extern const Variant g_variants_f16[];
+extern const int g_num_variants_f16;
+extern const Variant g_variants_bf16[];
+extern const int g_num_variants_bf16;
+extern const Variant g_variants_fp8[];
+extern const int g_num_variants_fp8;
+extern const Variant g_variants_fp4[];
+extern const int g_num_variants_fp4;
+
+}  // namespace tb

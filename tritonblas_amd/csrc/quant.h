@@ -1,0 +1,22 @@
+// Host/device shared declarations of the MXFP4 quantisation kernel.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tb {
+
+enum : int { QT_F16 = 0, QT_BF16 = 1, QT_F32 = 4 };  // same numbering as the public element types
+
+struct QuantParams {
+  const uint8_t* x;
+  uint8_t* codes;
+  uint8_t* scales;
+  int64_t m, n;
+  int64_t x_stride;       // elements
+  int64_t codes_stride;   // bytes
+  int64_t scales_stride;  // bytes
+};
+
+hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, hipStream_t stream);
+
+}  // namespace tb

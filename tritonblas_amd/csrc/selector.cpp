@@ -1,0 +1,139 @@
+// Analytical tile selector for the gfx950 kernel family: scores every built tile variant with a
+// small roofline-style model (MFMA issue time, LDS read time, L2->LDS fill time, wave quantisation
+// over the CUs, HBM time) and derives the launch parameters that go with the winner (GROUP_M, XCD
+// remap, Stream-K grid, work-stealing slots).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include "selector.h"
+
+namespace tb {
+
+static int type_bits(int t) {
+  switch (t) {
+    case TB_F16: case TB_BF16: return 16;
+    case TB_FP8_E4M3: return 8;
+    case TB_FP4_E2M1: return 4;
+    case TB_F32: return 32;
+  }
+  return 0;
+}
+
+// dense MFMA flops per clock per CU
+static double mfma_flops_per_clk(int t) {
+  switch (t) {
+    case TB_F16: case TB_BF16: return 4096.0;
+    case TB_FP8_E4M3: return 8192.0;
+    case TB_FP4_E2M1: return 16384.0;
+  }
+  return 1024.0;
+}
+
+void default_hw(tb_hw* hw) {
+  std::memset(hw, 0, sizeof(*hw));
+  hw->n_cu = 256; hw->num_xcd = 8; hw->cu_per_xcd = 32; hw->lds_bytes = 163840; hw->l2_bytes = 4 << 20;
+  hw->clock_khz = 2400000; hw->mem_clock_khz = 2000000; hw->wave_size = 64; hw->hbm_gbps = 8000.0;
+  std::strncpy(hw->arch, "gfx950", sizeof(hw->arch) - 1);
+}
+
+int ws_counters_per_xcd(int64_t total_tiles) {
+  if (total_tiles <= 512) return 8;
+  if (total_tiles <= 1536) return 4;
+  if (total_tiles <= 2048) return 2;
+  return 1;
+}
+
+static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Workgroups of one variant that fit a CU (LDS and wave slots), capped by what the kernel was built for.
+int variant_occupancy(const TileInfo& v, const tb_hw& hw) {
+  int by_lds = std::max(1, hw.lds_bytes / std::max(1, v.lds_bytes));
+  int by_waves = std::max(1, (8 * 4) / (v.threads / 64));
+  return std::max(1, std::min({by_lds, by_waves, v.minb}));
+}
+
+static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk, double* comp_us,
+                    double* mem_us) {
+  const double clk = hw.clock_khz * 1e3;
+  const int bits = type_bits(pr.a_type);
+  const double esz = bits / 8.0;
+  const int64_t tiles_m = cdiv(pr.m, v.bm), tiles_n = cdiv(pr.n, v.bn);
+  const int64_t tiles = tiles_m * tiles_n + (pr.num_groups > 0 ? pr.num_groups * tiles_n / 2 : 0);
+  const int64_t k_iters = cdiv(pr.k, v.bk);
+  const int occ = variant_occupancy(v, hw);
+  const int waves = v.threads / 64;
+  const double bkb = v.bk * esz;
+
+  // per K step, per workgroup (cycles)
+  const double t_mfma = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type);
+  const int wm = (v.bm >= v.bn) ? std::max(1, waves / 2) : 1;  // informational split, matches the built shapes
+  (void)wm;
+  const double wave_rows = (double)v.bm / 2 + (double)v.bn / 2;  // rows each of the 2x2 waves reads
+  const double t_lds = waves * wave_rows * bkb / 128.0;          // 128 B/clk/CU LDS read
+  const double t_fill = (v.bm + v.bn) * bkb / 64.0;              // L2 -> LDS, 64 B/clk/CU
+  const double t_sync = 120.0;
+  double t_iter;
+  if (occ >= 2) t_iter = std::max({t_mfma, t_lds, t_fill}) + t_sync / occ;   // workgroups overlap each other
+  else t_iter = std::max(t_mfma + 0.25 * t_lds, std::max(t_lds, t_fill)) + t_sync;
+  const double c_bytes = type_bits(pr.c_type) / 8.0;
+  const double t_epi = 1500.0 + v.bm * v.bn * c_bytes / 32.0;
+  const double t_tile = k_iters * t_iter + t_epi;
+
+  double cycles;
+  if (streamk) {
+    // iterations spread evenly over all resident workgroups, one fixup per workgroup
+    const double slots = (double)hw.n_cu * occ;
+    const double iters_per_wg = std::ceil((double)tiles * k_iters / slots);
+    cycles = iters_per_wg * t_iter * occ + t_epi * std::max(1.0, (double)tiles / slots) + 2000.0;
+  } else {
+    const double rounds = std::ceil((double)tiles / ((double)hw.n_cu * occ));
+    cycles = rounds * t_tile * occ;  // occ workgroups share the CU's MFMA/LDS throughput
+    if (occ >= 2) cycles = std::max(cycles, rounds * (k_iters * t_mfma * occ + t_epi));
+  }
+  *comp_us = cycles / clk * 1e6;
+
+  // HBM: every operand once, plus re-reads when a band of tiles does not stay in L2/MALL
+  const double a_bytes = (double)pr.m * pr.k * esz, b_bytes = (double)pr.n * pr.k * esz * std::max(1, pr.num_groups);
+  const double c_out = (double)pr.m * pr.n * c_bytes;
+  const double reread = 1.0 + 0.15 * std::max(0.0, std::log2((double)std::max<int64_t>(1, 256 / std::min(v.bm, v.bn))));
+  *mem_us = ((a_bytes + b_bytes) * reread + c_out) / (hw.hbm_gbps * 1e9 * 0.8) * 1e6;
+  return std::max(*comp_us, *mem_us) + 3.0;
+}
+
+int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out) {
+  int best = -1;
+  double best_t = 0, best_c = 0, best_m = 0;
+  for (int i = 0; i < ntiles; ++i) {
+    const TileInfo& v = tiles[i];
+    if (!v.fast) continue;  // the gather kernels are a fallback, never a choice of the model
+    if (v.lds_bytes > hw.lds_bytes) continue;
+    double c, m;
+    double t = score(pr, hw, v, pr.streamk != 0, &c, &m);
+    // prefer the larger tile on ties (less L2 traffic than the model resolves)
+    if (best < 0 || t < best_t * 0.995 || (t <= best_t * 1.005 && (int64_t)v.bm * v.bn > (int64_t)tiles[best].bm * tiles[best].bn)) {
+      best = i; best_t = t; best_c = c; best_m = m;
+    }
+  }
+  if (best < 0) return TB_ERR_BAD_TILE;
+  const TileInfo& v = tiles[best];
+  std::memset(out, 0, sizeof(*out));
+  out->block_m = v.bm; out->block_n = v.bn; out->block_k = v.bk;
+  const int64_t tiles_m = cdiv(pr.m, v.bm), tiles_n = cdiv(pr.n, v.bn);
+  const int64_t total = tiles_m * tiles_n;
+  out->group_m = (int)std::min<int64_t>(8, tiles_m);
+  out->num_xcds = hw.num_xcd;
+  out->occupancy = variant_occupancy(v, hw);
+  out->num_stages = v.stages;
+  out->lds_bytes = v.lds_bytes;
+  out->counters_per_xcd = ws_counters_per_xcd(total);
+  // Stream-K grid: every resident workgroup slot, but never more workgroups than K iterations to share
+  const int64_t k_iters = cdiv(pr.k, v.bk);
+  int64_t grid = (int64_t)hw.n_cu * out->occupancy;
+  grid = std::min(grid, total * k_iters);
+  if (total % grid == 0 && total >= grid) grid = std::min<int64_t>(grid, total);
+  out->sk_grid = (int)std::max<int64_t>(1, grid);
+  out->est_compute_us = best_c; out->est_memory_us = best_m; out->est_total_us = best_t;
+  return TB_OK;
+}
+
+}  // namespace tb

@@ -1,0 +1,17 @@
+// Host-only: analytical tile selector.
+#pragma once
+#include <stdint.h>
+#include "../../include/tritonblas_amd.h"
+
+namespace tb {
+
+struct TileInfo {
+  int dt, bm, bn, bk, threads, lds_bytes, minb, fast, stages;
+};
+
+void default_hw(tb_hw* hw);
+int ws_counters_per_xcd(int64_t total_tiles);
+int variant_occupancy(const TileInfo& v, const tb_hw& hw);
+int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out);
+
+}  // namespace tb

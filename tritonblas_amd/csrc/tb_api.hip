@@ -1,0 +1,433 @@
+// C ABI of the library: argument validation, kernel-variant choice and launches.
+// No device allocation, no synchronisation, no exceptions: every entry point returns a status.
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <vector>
+#include "../../include/tritonblas_amd.h"
+#include "gemm_variants.h"
+#include "quant.h"
+#include "selector.h"
+
+using namespace tb;
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+tb_hw g_hw[MAX_DEVICES];
+std::once_flag g_hw_once[MAX_DEVICES];
+int g_hw_status[MAX_DEVICES];
+
+int read_num_xcc(int n_cu, const char* arch) {
+  // KFD reports the XCC count per node; fall back to what the known parts have.
+  if (std::strncmp(arch, "gfx950", 6) == 0) return n_cu >= 64 ? std::max(1, n_cu / 32) : 1;
+  if (std::strncmp(arch, "gfx942", 6) == 0) {
+    if (n_cu == 304) return 8;
+    if (n_cu == 228) return 6;
+    return std::max(1, n_cu / 38);
+  }
+  return 1;
+}
+
+void query_hw(int dev) {
+  hipDeviceProp_t pr;
+  if (hipGetDeviceProperties(&pr, dev) != hipSuccess) { g_hw_status[dev] = TB_ERR_NO_DEVICE; return; }
+  tb_hw hw;
+  default_hw(&hw);
+  hw.n_cu = pr.multiProcessorCount;
+  std::memset(hw.arch, 0, sizeof(hw.arch));
+  for (int i = 0; i < (int)sizeof(hw.arch) - 1 && pr.gcnArchName[i] && pr.gcnArchName[i] != ':'; ++i) hw.arch[i] = pr.gcnArchName[i];
+  hw.num_xcd = read_num_xcc(hw.n_cu, hw.arch);
+  hw.cu_per_xcd = std::max(1, hw.n_cu / hw.num_xcd);
+  hw.lds_bytes = (int)pr.maxSharedMemoryPerMultiProcessor;
+  hw.l2_bytes = pr.l2CacheSize;
+  hw.clock_khz = pr.clockRate;
+  hw.mem_clock_khz = pr.memoryClockRate;
+  hw.wave_size = pr.warpSize;
+  // HBM3E: bus width (bits) x memory clock x 2 (DDR) / 8; the runtime reports the command clock
+  double gbps = (double)pr.memoryBusWidth / 8.0 * (double)pr.memoryClockRate * 1e3 * 2.0 / 1e9;
+  hw.hbm_gbps = (gbps > 100.0) ? gbps : 8000.0;
+  if (std::strncmp(hw.arch, "gfx950", 6) == 0) hw.hbm_gbps = 8000.0;
+  g_hw[dev] = hw;
+  g_hw_status[dev] = TB_OK;
+}
+
+int current_hw(tb_hw* out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return TB_ERR_NO_DEVICE;
+  std::call_once(g_hw_once[dev], query_hw, dev);
+  if (g_hw_status[dev] != TB_OK) return g_hw_status[dev];
+  *out = g_hw[dev];
+  return TB_OK;
+}
+
+void variant_table(int dt, const Variant** v, int* n) {
+  switch (dt) {
+    case TB_F16: *v = g_variants_f16; *n = g_num_variants_f16; break;
+    case TB_BF16: *v = g_variants_bf16; *n = g_num_variants_bf16; break;
+    case TB_FP8_E4M3: *v = g_variants_fp8; *n = g_num_variants_fp8; break;
+    case TB_FP4_E2M1: *v = g_variants_fp4; *n = g_num_variants_fp4; break;
+    default: *v = nullptr; *n = 0;
+  }
+}
+
+// distinct tiles (layout-independent) of one element type, fast kernels first
+std::vector<TileInfo> tile_infos(int dt) {
+  const Variant* v; int n;
+  variant_table(dt, &v, &n);
+  std::vector<TileInfo> out;
+  for (int i = 0; i < n; ++i) {
+    bool seen = false;
+    for (auto& t : out) seen |= (t.bm == v[i].bm && t.bn == v[i].bn && t.bk == v[i].bk && t.fast == v[i].fast);
+    if (!seen) out.push_back(TileInfo{v[i].dt, v[i].bm, v[i].bn, v[i].bk, v[i].threads, v[i].lds_bytes, v[i].minb, v[i].fast, v[i].stages});
+  }
+  return out;
+}
+
+const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast) {
+  const Variant* v; int n;
+  variant_table(dt, &v, &n);
+  for (int i = 0; i < n; ++i)
+    if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk)))
+      return &v[i];
+  return nullptr;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : 1; }
+int c_bytes(int t) { return t == TB_F32 ? 4 : 2; }
+
+// Everything the launch path needs, independent of which public descriptor it came from.
+struct Job {
+  int dt = 0, c_type = 0, bias_type = 0;
+  int64_t M = 0, N = 0, K = 0;
+  const void* A = nullptr; const void* B = nullptr; void* C = nullptr;
+  int64_t a_sr = 0, a_sk = 0, b_sr = 0, b_sk = 0;  // storage units: row = m (A) / n (B)
+  int64_t c_sm = 0, c_sn = 0;
+  const float* sa = nullptr; const float* sb = nullptr;
+  const void* bias = nullptr; int64_t bias_stride = 0;
+  const void* mxa = nullptr; const void* mxb = nullptr;
+  int64_t mxa_sr = 0, mxa_sk = 0, mxb_sr = 0, mxb_sk = 0;
+  int bm = 0, bn = 0, bk = 0, group_m = 0, num_xcds = 0;
+  int schedule = TB_SCHED_PERSISTENT, grid = 0, counters_per_xcd = 0;
+  void* workspace = nullptr; size_t workspace_bytes = 0;
+  uint32_t epoch = 1, spin_limit = 0;
+  // grouped
+  const int32_t* group_offsets = nullptr; int num_groups = 0;
+  int64_t b_group_stride = 0, sb_group_stride = 0;
+};
+
+struct Plan {
+  const Variant* v = nullptr;
+  GemmParams p;
+  int grid = 0;
+  size_t ws_need = 0, ws_flags_off = 0, ws_p_off = 0, ws_counters_off = 0;
+};
+
+int kernel_occupancy(const Variant* v) {
+  static std::mutex mu;
+  static std::vector<std::pair<const void*, int>> cache;
+  std::lock_guard<std::mutex> lk(mu);
+  for (auto& c : cache) if (c.first == v->kernel) return c.second;
+  int nb = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->kernel, v->threads, 0) != hipSuccess || nb < 1) nb = 1;
+  cache.emplace_back(v->kernel, nb);
+  return nb;
+}
+
+int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
+  if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
+  if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
+  if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32) return TB_ERR_BAD_DTYPE;
+  const int usz = unit_bytes(j.dt);
+  const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
+  if (j.K % epu) return TB_ERR_BAD_SHAPE;
+  const int64_t KU = j.K / epu;
+
+  // which loader can address each operand
+  auto k_major_ok = [&](const void* ptr, int64_t s_row, int64_t s_k, int64_t rows) {
+    return s_k == 1 && aligned16(ptr) && (rows == 1 || (s_row * usz) % 16 == 0) && s_row >= 0;
+  };
+  auto m_major_ok = [&](const void* ptr, int64_t s_row, int64_t s_k, int64_t rows) {
+    return usz == 2 && s_row == 1 && aligned16(ptr) && (s_k * usz) % 16 == 0 && rows % 8 == 0 && j.num_groups == 0;
+  };
+  int alay = -1, blay = -1;
+  if (k_major_ok(j.A, j.a_sr, j.a_sk, j.M)) alay = LAY_K; else if (m_major_ok(j.A, j.a_sr, j.a_sk, j.M)) alay = LAY_M;
+  if (k_major_ok(j.B, j.b_sr, j.b_sk, j.N)) blay = LAY_K; else if (m_major_ok(j.B, j.b_sr, j.b_sk, j.N)) blay = LAY_M;
+
+  // tile
+  int bm = j.bm, bn = j.bn, bk = j.bk;
+  tb_selection sel;
+  std::memset(&sel, 0, sizeof(sel));
+  if (bm == 0 || bn == 0 || bk == 0) {
+    tb_problem pr;
+    std::memset(&pr, 0, sizeof(pr));
+    pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+    pr.a_k_contiguous = alay == LAY_K; pr.b_k_contiguous = blay == LAY_K;
+    pr.streamk = j.schedule == TB_SCHED_STREAMK; pr.num_groups = j.num_groups;
+    auto infos = tile_infos(j.dt);
+    int st = select_tile(pr, hw, infos.data(), (int)infos.size(), &sel);
+    if (st != TB_OK) return st;
+    bm = sel.block_m; bn = sel.block_n; bk = sel.block_k;
+  }
+  const Variant* v = nullptr;
+  bool fast = alay >= 0 && blay >= 0 && (KU % (bk / epu) == 0);
+  if (fast) {
+    // 32-bit offsets inside a tile
+    if ((alay == LAY_K && (int64_t)bm * j.a_sr * usz >= (1ll << 31)) || (blay == LAY_K && (int64_t)bn * j.b_sr * usz >= (1ll << 31)) ||
+        (alay == LAY_M && (int64_t)bk * j.a_sk * usz >= (1ll << 31)) || (blay == LAY_M && (int64_t)bk * j.b_sk * usz >= (1ll << 31)))
+      fast = false;
+  }
+  if (fast) {
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1);
+    if (!v) return TB_ERR_BAD_TILE;
+  } else {
+    if (j.bm != 0) {
+      // an explicit tile must at least name a built one, even when the gather kernel runs instead
+      bool known = false;
+      for (auto& t : tile_infos(j.dt)) known |= (t.bm == bm && t.bn == bn && t.bk == bk);
+      if (!known) return TB_ERR_BAD_TILE;
+    }
+    v = find_variant(j.dt, 0, 0, 0, LAY_K, LAY_K, 0);
+    if (!v) return TB_ERR_BAD_LAYOUT;
+  }
+  if (j.dt == TB_FP4_E2M1 && (j.a_sk != 1 || j.b_sk != 1)) return TB_ERR_BAD_LAYOUT;
+
+  GemmParams& p = plan->p;
+  std::memset(&p, 0, sizeof(p));
+  p.A = (const uint8_t*)j.A; p.B = (const uint8_t*)j.B; p.C = (uint8_t*)j.C;
+  p.sa = j.sa; p.sb = j.sb; p.bias = (const uint8_t*)j.bias;
+  p.mxa = (const uint8_t*)j.mxa; p.mxb = (const uint8_t*)j.mxb;
+  p.M = (int32_t)j.M; p.N = (int32_t)j.N; p.KU = KU;
+  p.a_sr = j.a_sr; p.a_sk = j.a_sk; p.b_sr = j.b_sr; p.b_sk = j.b_sk;
+  p.c_sm = j.c_sm; p.c_sn = j.c_sn;
+  p.mxa_sr = j.mxa_sr; p.mxa_sk = j.mxa_sk; p.mxb_sr = j.mxb_sr; p.mxb_sk = j.mxb_sk;
+  p.bias_stride = j.bias_stride; p.c_type = j.c_type; p.bias_type = j.bias_type;
+  p.a_vec = p.b_vec = v->fast;
+  const int cb = c_bytes(j.c_type);
+  p.c_vec = (j.c_sn == 1 && (j.c_sm % 4 == 0 || j.M == 1) && ((uintptr_t)j.C % (4 * cb)) == 0) ? 1 : 0;
+  if (j.dt == TB_FP4_E2M1) {
+    const int ksub = v->bk / 128;
+    p.mx_vec = (j.mxa_sk == 1 && j.mxb_sk == 1 && j.mxa_sr % ksub == 0 && j.mxb_sr % ksub == 0 &&
+                ((uintptr_t)j.mxa % ksub) == 0 && ((uintptr_t)j.mxb % ksub) == 0) ? 1 : 0;
+  }
+  p.tiles_m = (int32_t)((j.M + v->bm - 1) / v->bm);
+  p.tiles_n = (int32_t)((j.N + v->bn - 1) / v->bn);
+  const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+  if (total > INT32_MAX) return TB_ERR_BAD_SHAPE;
+  p.total_tiles = (int32_t)total;
+  p.k_iters = (int32_t)((j.K + v->bk - 1) / v->bk);
+  p.group_m = j.group_m > 0 ? j.group_m : std::min(8, (int)p.tiles_m);
+  p.num_xcds = j.num_xcds > 0 ? j.num_xcds : hw.num_xcd;
+  p.epoch = j.epoch; p.spin_limit = j.spin_limit ? j.spin_limit : (1u << 24);
+  p.group_offsets = j.group_offsets; p.num_groups = j.num_groups;
+  p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
+
+  const int occ = need_device ? kernel_occupancy(v) : std::max(1, std::min(v->minb, hw.lds_bytes / v->lds_bytes));
+  const int resident = hw.n_cu * occ;
+  int grid;
+  plan->ws_need = 0;
+  if (j.num_groups > 0) {
+    p.mode = MODE_GROUPED;
+    grid = (int)(((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n);
+  } else if (j.schedule == TB_SCHED_PERSISTENT) {
+    p.mode = MODE_STATIC;
+    grid = p.total_tiles;
+  } else if (j.schedule == TB_SCHED_WORK_STEALING) {
+    p.mode = MODE_WS;
+    grid = j.grid > 0 ? j.grid : resident;
+    p.counters_per_xcd = j.counters_per_xcd > 0 ? j.counters_per_xcd : ws_counters_per_xcd(total);
+    plan->ws_counters_off = CTL_WORDS * 4;
+    plan->ws_need = plan->ws_counters_off + (size_t)p.num_xcds * p.counters_per_xcd * COUNTER_STRIDE * 4;
+  } else if (j.schedule == TB_SCHED_STREAMK) {
+    p.mode = MODE_SK;
+    int64_t g = j.grid > 0 ? j.grid : std::min<int64_t>(resident, total * p.k_iters);
+    if (g > resident) return TB_ERR_BAD_SCHEDULE;  // owners spin on later workgroups: all must be resident
+    grid = (int)g;
+    p.sk_tiles = (int32_t)(total % grid);
+    plan->ws_flags_off = CTL_WORDS * 4;
+    plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
+    plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
+  } else {
+    return TB_ERR_BAD_SCHEDULE;
+  }
+  if (grid <= 0) return TB_ERR_BAD_SHAPE;
+  p.chunk = std::min(p.group_m * p.group_m, std::max(1, grid / p.num_xcds));
+  plan->grid = grid;
+  plan->v = v;
+  return TB_OK;
+}
+
+int launch(const Job& j, hipStream_t stream) {
+  tb_hw hw;
+  int st = current_hw(&hw);
+  if (st != TB_OK) return st;
+  Plan plan;
+  st = make_plan(j, hw, true, &plan);
+  if (st != TB_OK) return st;
+  GemmParams& p = plan.p;
+  if (plan.ws_need) {
+    if (!j.workspace || j.workspace_bytes < plan.ws_need || ((uintptr_t)j.workspace & 255)) return TB_ERR_WORKSPACE;
+    uint8_t* ws = (uint8_t*)j.workspace;
+    p.ctl = (uint32_t*)ws;
+    if (p.mode == MODE_WS) p.counters = (int32_t*)(ws + plan.ws_counters_off);
+    if (p.mode == MODE_SK) { p.flags = (uint32_t*)(ws + plan.ws_flags_off); p.P = (float*)(ws + plan.ws_p_off); }
+  }
+  void* args[] = {(void*)&p};
+  hipError_t e = hipLaunchKernel(plan.v->kernel, dim3((unsigned)plan.grid), dim3((unsigned)plan.v->threads), args, 0, stream);
+  if (e != hipSuccess) { (void)hipGetLastError(); return TB_ERR_LAUNCH; }
+  return TB_OK;
+}
+
+int job_from_gemm(const tb_gemm_desc* d, Job* j) {
+  if (!d) return TB_ERR_NULL_POINTER;
+  if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
+  if (d->a_type != d->b_type) return TB_ERR_BAD_DTYPE;
+  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3) return TB_ERR_BAD_DTYPE;
+  if ((d->a_scale == nullptr) != (d->b_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
+  if (d->bias && d->bias_type != TB_F16 && d->bias_type != TB_BF16 && d->bias_type != TB_F32) return TB_ERR_BAD_DTYPE;
+  j->dt = d->a_type; j->c_type = d->c_type; j->bias_type = d->bias_type;
+  j->M = d->m; j->N = d->n; j->K = d->k;
+  j->A = d->a; j->B = d->b; j->C = d->c;
+  j->a_sr = d->a_stride_m; j->a_sk = d->a_stride_k; j->b_sr = d->b_stride_n; j->b_sk = d->b_stride_k;
+  j->c_sm = d->c_stride_m; j->c_sn = d->c_stride_n;
+  j->sa = d->a_scale; j->sb = d->b_scale; j->bias = d->bias; j->bias_stride = d->bias_stride;
+  j->bm = d->block_m; j->bn = d->block_n; j->bk = d->block_k; j->group_m = d->group_m; j->num_xcds = d->num_xcds;
+  j->schedule = d->schedule; j->grid = d->grid; j->counters_per_xcd = d->counters_per_xcd;
+  j->workspace = d->workspace; j->workspace_bytes = d->workspace_bytes; j->epoch = d->epoch; j->spin_limit = d->spin_limit;
+  return TB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tb_abi_version(void) { return TB_ABI_VERSION; }
+
+const char* tb_status_string(int status) {
+  switch (status) {
+    case TB_OK: return "ok";
+    case TB_ERR_NULL_POINTER: return "null pointer";
+    case TB_ERR_BAD_SHAPE: return "Incompatible Dimensions";
+    case TB_ERR_BAD_DTYPE: return "unsupported element type";
+    case TB_ERR_BAD_LAYOUT: return "unsupported strides";
+    case TB_ERR_BAD_TILE: return "no kernel variant for this tile";
+    case TB_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case TB_ERR_BAD_SCHEDULE: return "invalid schedule or grid";
+    case TB_ERR_LAUNCH: return "kernel launch failed";
+    case TB_ERR_NO_DEVICE: return "no usable HIP device";
+    case TB_ERR_BAD_ARGUMENT: return "bad argument";
+  }
+  return "unknown status";
+}
+
+int tb_device_info(int device, tb_hw* out) {
+  if (!out) return TB_ERR_NULL_POINTER;
+  if (device < 0) { default_hw(out); return TB_OK; }
+  if (device >= MAX_DEVICES) return TB_ERR_BAD_ARGUMENT;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || device >= count) { (void)hipGetLastError(); return TB_ERR_NO_DEVICE; }
+  std::call_once(g_hw_once[device], query_hw, device);
+  if (g_hw_status[device] != TB_OK) return g_hw_status[device];
+  *out = g_hw[device];
+  return TB_OK;
+}
+
+int tb_list_tiles(int32_t a_type, int32_t* triples, int32_t cap) {
+  auto infos = tile_infos(a_type);
+  int n = 0;
+  for (auto& t : infos) {
+    if (!t.fast) continue;
+    if (triples && n < cap) { triples[3 * n] = t.bm; triples[3 * n + 1] = t.bn; triples[3 * n + 2] = t.bk; }
+    ++n;
+  }
+  return n;
+}
+
+int tb_select(const tb_problem* problem, const tb_hw* hw, tb_selection* out) {
+  if (!problem || !out) return TB_ERR_NULL_POINTER;
+  if (problem->m <= 0 || problem->n <= 0 || problem->k <= 0) return TB_ERR_BAD_SHAPE;
+  tb_hw local;
+  if (hw) local = *hw; else default_hw(&local);
+  auto infos = tile_infos(problem->a_type);
+  if (infos.empty()) return TB_ERR_BAD_DTYPE;
+  return select_tile(*problem, local, infos.data(), (int)infos.size(), out);
+}
+
+int tb_gemm(const tb_gemm_desc* desc, void* stream) {
+  Job j;
+  int st = job_from_gemm(desc, &j);
+  if (st != TB_OK) return st;
+  if (!j.A || !j.B || !j.C) return TB_ERR_NULL_POINTER;
+  return launch(j, (hipStream_t)stream);
+}
+
+size_t tb_workspace_bytes(const tb_gemm_desc* desc) {
+  Job j;
+  if (job_from_gemm(desc, &j) != TB_OK) return 0;
+  tb_hw hw;
+  bool have_dev = current_hw(&hw) == TB_OK;
+  if (!have_dev) default_hw(&hw);
+  // alignment of the real pointers decides the kernel family; with null pointers assume aligned
+  Plan plan;
+  if (make_plan(j, hw, have_dev, &plan) != TB_OK) return 0;
+  return plan.ws_need;
+}
+
+int tb_gemm_fp4(const tb_gemm_fp4_desc* d, void* stream) {
+  if (!d) return TB_ERR_NULL_POINTER;
+  if (d->struct_bytes != sizeof(tb_gemm_fp4_desc)) return TB_ERR_BAD_ARGUMENT;
+  if (!d->a || !d->b || !d->c || !d->a_scales || !d->b_scales) return TB_ERR_NULL_POINTER;
+  if (d->k <= 0 || d->k % 32) return TB_ERR_BAD_SHAPE;
+  Job j;
+  j.dt = TB_FP4_E2M1; j.c_type = d->c_type;
+  j.M = d->m; j.N = d->n; j.K = d->k;
+  j.A = d->a; j.B = d->b; j.C = d->c;
+  j.a_sr = d->a_stride_m; j.a_sk = 1; j.b_sr = d->b_stride_n; j.b_sk = 1;
+  j.c_sm = d->c_stride_m; j.c_sn = d->c_stride_n;
+  j.mxa = d->a_scales; j.mxb = d->b_scales;
+  j.mxa_sr = d->a_scales_stride_m; j.mxa_sk = d->a_scales_stride_k;
+  j.mxb_sr = d->b_scales_stride_n; j.mxb_sk = d->b_scales_stride_k;
+  j.bm = d->block_m; j.bn = d->block_n; j.bk = d->block_k; j.group_m = d->group_m; j.num_xcds = d->num_xcds;
+  return launch(j, (hipStream_t)stream);
+}
+
+int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
+  if (!d) return TB_ERR_NULL_POINTER;
+  if (d->struct_bytes != sizeof(tb_grouped_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
+  if (!d->a || !d->w || !d->c || !d->group_offsets) return TB_ERR_NULL_POINTER;
+  if ((d->a_scale == nullptr) != (d->w_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
+  if (d->num_groups <= 0) return TB_ERR_BAD_SHAPE;
+  Job j;
+  j.dt = TB_FP8_E4M3; j.c_type = d->c_type;
+  j.M = d->m_total; j.N = d->n; j.K = d->k;
+  j.A = d->a; j.B = d->w; j.C = d->c;
+  j.a_sr = d->a_stride_m; j.a_sk = 1; j.b_sr = d->w_stride_n; j.b_sk = 1;
+  j.c_sm = d->c_stride_m; j.c_sn = d->c_stride_n;
+  j.sa = d->a_scale; j.sb = d->w_scale;
+  j.bm = d->block_m; j.bn = d->block_n; j.bk = d->block_k; j.group_m = d->group_m; j.num_xcds = d->num_xcds;
+  j.group_offsets = d->group_offsets; j.num_groups = d->num_groups;
+  j.b_group_stride = d->w_stride_g; j.sb_group_stride = d->n;
+  if ((d->w_stride_g * 1) % 16) return TB_ERR_BAD_LAYOUT;
+  return launch(j, (hipStream_t)stream);
+}
+
+int tb_hadamard_mxfp4_quant(const tb_quant_desc* d, void* stream) {
+  if (!d) return TB_ERR_NULL_POINTER;
+  if (d->struct_bytes != sizeof(tb_quant_desc)) return TB_ERR_BAD_ARGUMENT;
+  if (!d->x || !d->codes || !d->scales) return TB_ERR_NULL_POINTER;
+  if (d->m <= 0 || d->n <= 0 || d->n % 32) return TB_ERR_BAD_SHAPE;
+  if (d->x_type != TB_F16 && d->x_type != TB_BF16 && d->x_type != TB_F32) return TB_ERR_BAD_DTYPE;
+  const int xb = d->x_type == TB_F32 ? 4 : 2;
+  if (!aligned16(d->x) || (d->x_stride_m * xb) % 16 || ((uintptr_t)d->codes & 3) || d->codes_stride_m % 4) return TB_ERR_BAD_LAYOUT;
+  QuantParams p;
+  p.x = (const uint8_t*)d->x; p.codes = (uint8_t*)d->codes; p.scales = (uint8_t*)d->scales;
+  p.m = d->m; p.n = d->n; p.x_stride = d->x_stride_m; p.codes_stride = d->codes_stride_m; p.scales_stride = d->scales_stride_m;
+  hipError_t e = launch_quant(p, d->x_type, d->hadamard != 0, (hipStream_t)stream);
+  if (e != hipSuccess) return TB_ERR_LAUNCH;
+  return TB_OK;
+}
+
+}  // extern "C"

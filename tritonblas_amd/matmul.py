@@ -1,0 +1,289 @@
+"""GEMM entry points with the reference's Python signatures (include/tritonblas/matmul.py).
+
+Each launcher fills one C descriptor and calls the shared library on torch's current stream; nothing
+here computes.  ``a`` is (M, K), ``b`` is (K, N) with arbitrary 2-D strides (transposes are views),
+``c`` is written in place and returned.
+"""
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import C
+from .config import MatmulConfig, matmul_preamble
+from .origami import OrigamiMatmulSelector
+
+
+def _make_matmul_selector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=0, streamk=False,
+                          num_stages: int = 2):
+    """Reference matmul.py:42-66."""
+    return OrigamiMatmulSelector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=mx_block_size,
+                                 streamk=streamk, num_stages=num_stages)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _check_device(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("tritonblas_amd: tensors must live on a GPU (there is no CPU path)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("tritonblas_amd: tensors are on different devices")
+    return dev
+
+
+def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b_scale=None, sk_grid=None):
+    assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
+    M, K = a.shape
+    _, N = b.shape
+    assert c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
+    dev = _check_device(a, b, c, bias, a_scale, b_scale)
+    lib = _lib.load()
+    d = _lib.tb_gemm_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+    d.a_type, d.b_type, d.c_type = _lib.tb_dtype(a.dtype), _lib.tb_dtype(b.dtype), _lib.tb_dtype(c.dtype)
+    d.m, d.n, d.k = M, N, K
+    d.a_stride_m, d.a_stride_k = a.stride(0), a.stride(1)
+    d.b_stride_k, d.b_stride_n = b.stride(0), b.stride(1)
+    d.c_stride_m, d.c_stride_n = c.stride(0), c.stride(1)
+    d.a, d.b, d.c = _ptr(a), _ptr(b), _ptr(c)
+    if a_scale is not None:
+        if a_scale.dtype != torch.float32 or b_scale.dtype != torch.float32:
+            raise RuntimeError("tritonblas_amd: scales must be float32")
+        a_scale, b_scale = a_scale.reshape(-1), b_scale.reshape(-1)
+        if not (a_scale.is_contiguous() and b_scale.is_contiguous() and a_scale.numel() == M and b_scale.numel() == N):
+            raise RuntimeError("tritonblas_amd: a_scale must be contiguous (M,) and b_scale contiguous (N,)")
+        d.a_scale, d.b_scale = _ptr(a_scale), _ptr(b_scale)
+    if bias is not None:
+        if bias.numel() != N:
+            raise AssertionError("Incompatible Dimensions")
+        d.bias, d.bias_type, d.bias_stride = _ptr(bias), _lib.tb_dtype(bias.dtype), bias.stride(0)
+    if selector is not None:
+        d.block_m, d.block_n, d.block_k = selector.block_m, selector.block_n, selector.block_k
+        d.group_m, d.num_xcds = selector.group_m, selector.num_sms
+        d.counters_per_xcd = selector.COUNTERS_PER_XCD
+    d.schedule = schedule
+    if schedule == _lib.TB_SCHED_STREAMK:
+        if sk_grid is not None:
+            d.grid = int(sk_grid)
+        elif selector is not None and selector.streamk:
+            d.grid = selector.sk_grid
+    if schedule != _lib.TB_SCHED_PERSISTENT:
+        need = lib.tb_workspace_bytes(d)
+        if need == 0:
+            # the descriptor was refused; run the launch to surface the status
+            _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
+        if config is None:
+            config = MatmulConfig(device=dev, workspace=None, selector=selector)
+        ws = config.ensure(need)
+        d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
+        d.epoch = config.next_epoch()
+    with torch.cuda.device(dev):
+        _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
+    return c
+
+
+def persistent_matmul_lt(a, b, c, selector, config: Optional[MatmulConfig] = None, bias=None, a_scale=None,
+                         b_scale=None, quantized: bool = False, work_stealing: bool = False):
+    """Data-parallel launch, optionally through the work-stealing queues (reference matmul.py:69-200)."""
+    sched = _lib.TB_SCHED_WORK_STEALING if (work_stealing and config is not None) else _lib.TB_SCHED_PERSISTENT
+    return _launch_gemm(a, b, c, selector, config, sched, bias=bias,
+                        a_scale=a_scale if quantized else None, b_scale=b_scale if quantized else None)
+
+
+def streamk_matmul_lt(a, b, c, selector, config: Optional[MatmulConfig] = None, bias=None, sk_grid=None,
+                      a_scale=None, b_scale=None, quantized: bool = False, work_stealing: bool = False):
+    """Stream-K launch (reference matmul.py:202-366).  ``work_stealing`` only changes the grid in the
+    reference (grid = CU count); here the Stream-K grid already fills the device."""
+    return _launch_gemm(a, b, c, selector, config, _lib.TB_SCHED_STREAMK, bias=bias, sk_grid=sk_grid,
+                        a_scale=a_scale if quantized else None, b_scale=b_scale if quantized else None)
+
+
+def matmul_lt(a, b, c, selector, config: MatmulConfig = None, enable_streamk=False, work_stealing=False):
+    """Reference matmul.py:368-378."""
+    assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
+    if enable_streamk:
+        return streamk_matmul_lt(a, b, c, selector, config, work_stealing=work_stealing)
+    return persistent_matmul_lt(a, b, c, selector, config, work_stealing=work_stealing)
+
+
+def matmul_a8w8_lt(a, b, a_scale, b_scale, c, selector, config: MatmulConfig = None, enable_streamk=False,
+                   work_stealing=False):
+    """Reference matmul.py:380-390."""
+    assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
+    if enable_streamk:
+        return streamk_matmul_lt(a, b, c, selector, config, a_scale=a_scale, b_scale=b_scale, quantized=True)
+    return persistent_matmul_lt(a, b, c, selector, config, a_scale=a_scale, b_scale=b_scale, quantized=True,
+                                work_stealing=work_stealing)
+
+
+def _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, out_dtype_for_selector):
+    M, K = a.shape
+    _, N = b.shape
+    selector = _make_matmul_selector(M, N, K, a.dtype, b.dtype, out_dtype_for_selector, a.device,
+                                     streamk=bool(enable_streamk))
+    config = matmul_preamble(selector, a.device) if work_stealing else None
+    if enable_streamk:
+        return streamk_matmul_lt(a, b, out, selector, config, bias=bias, sk_grid=sk_grid, work_stealing=work_stealing)
+    return persistent_matmul_lt(a, b, out, selector, config, bias=bias, work_stealing=work_stealing)
+
+
+class _MatmulFn(torch.autograd.Function):
+    """Forward through the library, backward as two more library GEMMs (reference matmul.py:393-448)."""
+
+    @staticmethod
+    def forward(ctx, a, b, enable_streamk, sk_grid, work_stealing):
+        assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+        out = a.new_empty(a.shape[0], b.shape[1])
+        _run(a.detach(), b.detach(), out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
+        ctx.save_for_backward(a, b)
+        ctx.opts = (enable_streamk, sk_grid, work_stealing)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b = ctx.saved_tensors
+        sk, grid, ws = ctx.opts
+        g = grad_output.contiguous()
+        grad_a = matmul(g, b.detach().T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+        grad_b = matmul(a.detach().T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+        return grad_a, grad_b, None, None, None
+
+
+class _AddmmFn(torch.autograd.Function):
+    """Reference matmul.py:628-696."""
+
+    @staticmethod
+    def forward(ctx, bias, a, b, enable_streamk, sk_grid, work_stealing):
+        assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+        out = a.new_empty(a.shape[0], b.shape[1])
+        _run(a.detach(), b.detach(), out, bias.detach(), enable_streamk, sk_grid, work_stealing, bias.dtype)
+        ctx.save_for_backward(a, b)
+        ctx.opts = (enable_streamk, sk_grid, work_stealing)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        a, b = ctx.saved_tensors
+        sk, grid, ws = ctx.opts
+        g = grad_output.contiguous()
+        grad_a = matmul(g, b.detach().T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+        grad_b = matmul(a.detach().T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+        return grad_output.sum(dim=0), grad_a, grad_b, None, None, None
+
+
+def matmul(a, b, out: Optional[torch.Tensor] = None, enable_streamk: Optional[bool] = False,
+           sk_grid: Optional[int] = None, work_stealing: Optional[bool] = False) -> Optional[torch.Tensor]:
+    """Reference matmul.py:475-495: out=None allocates and supports autograd; out=... writes in
+    place, returns None and refuses tensors that require grad."""
+    if out is None:
+        return _MatmulFn.apply(a, b, enable_streamk, sk_grid, work_stealing)
+    if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad or out.requires_grad):
+        raise RuntimeError(
+            "tritonblas.matmul(): functions with out=... arguments don't support "
+            "automatic differentiation, but one of the arguments requires grad."
+        )
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    _run(a, b, out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
+    return None
+
+
+def addmm(bias, a, b, out: Optional[torch.Tensor] = None, enable_streamk: Optional[bool] = False,
+          sk_grid: Optional[int] = None, work_stealing: Optional[bool] = False) -> Optional[torch.Tensor]:
+    """Reference matmul.py:727-752; the bias is added per output column."""
+    if out is None:
+        return _AddmmFn.apply(bias, a, b, enable_streamk, sk_grid, work_stealing)
+    if torch.is_grad_enabled() and (bias.requires_grad or a.requires_grad or b.requires_grad or out.requires_grad):
+        raise RuntimeError(
+            "tritonblas.addmm(): functions with out=... arguments don't support "
+            "automatic differentiation, but one of the arguments requires grad."
+        )
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, bias.dtype)
+    return None
+
+
+def matmul_a8w8(a, b, a_scale, b_scale, c, enable_streamk=False, work_stealing=False, sk_grid=None):
+    """Reference matmul.py:498-517."""
+    assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
+    M, K = a.shape
+    _, N = b.shape
+    selector = _make_matmul_selector(M, N, K, a.dtype, b.dtype, c.dtype, a.device, streamk=bool(enable_streamk))
+    config = matmul_preamble(selector, a.device) if work_stealing else None
+    if enable_streamk:
+        return streamk_matmul_lt(a, b, c, selector, config, sk_grid=sk_grid, a_scale=a_scale, b_scale=b_scale,
+                                 quantized=True, work_stealing=work_stealing)
+    return persistent_matmul_lt(a, b, c, selector, config, a_scale=a_scale, b_scale=b_scale, quantized=True,
+                                work_stealing=work_stealing)
+
+
+def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = None, block_k: int = None,
+               group_size_m: int = 8, num_warps: int = 8, num_stages: int = 2):
+    """MXFP4 GEMM (reference matmul.py:519-625).  a: (M, K/2) uint8, b: (N, K/2) uint8 (two e2m1
+    codes per byte, low nibble first), scales (M|N, K/32) E8M0 bytes, c: (M, N) bf16/fp16.
+    ``num_warps``/``num_stages`` are accepted for signature compatibility; the kernels fix them."""
+    M, Kp = a.shape
+    N = b.shape[0]
+    K = Kp * 2
+    assert b.shape[1] * 2 == K, f"Incompatible Dimensions: A has K={K}, B has K={b.shape[1] * 2}"
+    dev = _check_device(a, b, c, a_scales, b_scales)
+    a, b = a.view(torch.uint8), b.view(torch.uint8)
+    a_scales, b_scales = a_scales.view(torch.uint8), b_scales.view(torch.uint8)
+    if a.stride(1) != 1 or b.stride(1) != 1:
+        raise RuntimeError("tritonblas_amd: matmul_fp4 needs K-contiguous packed operands")
+    d = _lib.tb_gemm_fp4_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_fp4_desc)
+    d.c_type = _lib.tb_dtype(c.dtype)
+    d.m, d.n, d.k = M, N, K
+    d.a, d.b, d.c = _ptr(a), _ptr(b), _ptr(c)
+    d.a_stride_m, d.b_stride_n = a.stride(0), b.stride(0)
+    d.c_stride_m, d.c_stride_n = c.stride(0), c.stride(1)
+    d.a_scales, d.b_scales = _ptr(a_scales), _ptr(b_scales)
+    d.a_scales_stride_m, d.a_scales_stride_k = a_scales.stride(0), a_scales.stride(1)
+    d.b_scales_stride_n, d.b_scales_stride_k = b_scales.stride(0), b_scales.stride(1)
+    if block_m is not None:
+        assert block_k % 64 == 0, "BLOCK_K must be multiple of 64 for FP4"
+        d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
+        d.group_m = group_size_m
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().tb_gemm_fp4(d, _lib.stream_handle(dev)), "tb_gemm_fp4")
+    return c
+
+
+def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int = None, block_n: int = None,
+                        block_k: int = None):
+    """Grouped (MoE) FP8 GEMM: rows ``group_offsets[e]:group_offsets[e+1]`` of ``a`` (M, K) meet expert
+    weight ``w[e]`` (N, K); ``c[rows] = cast((a[rows] @ w[e].T) * a_scale[rows, None] * w_scale[e][None, :])``.
+    ``group_offsets`` is an int32 device tensor of E+1 ascending row offsets.  One launch, no host sync."""
+    M, K = a.shape
+    E, N, K2 = w.shape
+    assert K == K2 and c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
+    assert group_offsets.numel() == E + 1 and group_offsets.dtype == torch.int32
+    dev = _check_device(a, w, c, a_scale, w_scale, group_offsets)
+    if a.stride(1) != 1 or w.stride(2) != 1:
+        raise RuntimeError("tritonblas_amd: grouped GEMM needs K-contiguous operands")
+    d = _lib.tb_grouped_gemm_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_grouped_gemm_desc)
+    d.c_type = _lib.tb_dtype(c.dtype)
+    d.m_total, d.n, d.k, d.num_groups = M, N, K, E
+    d.a, d.w, d.c = _ptr(a), _ptr(w), _ptr(c)
+    d.a_stride_m, d.w_stride_g, d.w_stride_n = a.stride(0), w.stride(0), w.stride(1)
+    d.c_stride_m, d.c_stride_n = c.stride(0), c.stride(1)
+    if a_scale is not None:
+        a_scale, w_scale = a_scale.reshape(-1), w_scale.reshape(E, N)
+        if not (a_scale.is_contiguous() and w_scale.is_contiguous()):
+            raise RuntimeError("tritonblas_amd: scales must be contiguous")
+        d.a_scale, d.w_scale = _ptr(a_scale), _ptr(w_scale)
+    d.group_offsets = _ptr(group_offsets)
+    if block_m is not None:
+        d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().tb_grouped_gemm_fp8(d, _lib.stream_handle(dev)), "tb_grouped_gemm_fp8")
+    return c
