@@ -1,0 +1,195 @@
+"""Headline benchmark: FP8 a8w8 GEMM 8192x28672x8192 (per-row / per-column scales, bf16 out) on one
+MI355X, plus the MXFP4 GEMM 8192x8192x16384, the fused Hadamard+MXFP4 quantiser and the other
+configurations as secondary figures on the same JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one launch of the FP8 GEMM with all operands resident in HBM.  The CPU baseline is
+torch.matmul in fp32 on the host cores over the dequantised operands of a bounded row slice.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp4": 10100.0}
+PEAK_HBM_GBPS = 8000.0
+
+
+def timed(fn, steps, warmup):
+    """K back-to-back launches between two events on the launch stream; returns ms per launch."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(end) / steps, wall_ms
+
+
+def fp8_inputs(m, n, k, dev, seed):
+    import tritonblas_amd.utils as U
+    g = torch.Generator(device=dev).manual_seed(seed)
+    a = torch.randn(m, k, device=dev, generator=g, dtype=torch.float32).bfloat16()
+    w = torch.randn(n, k, device=dev, generator=g, dtype=torch.float32).bfloat16()
+    aq, sa = U.quantize_tensor_per_channel(a, torch.float8_e4m3fn, axis=1)
+    wq, sw = U.quantize_tensor_per_channel(w, torch.float8_e4m3fn, axis=1)
+    del a, w
+    return aq, wq, sa, sw
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-secondary", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import tritonblas_amd as tb
+    import tritonblas_amd.utils as U
+    from oracle import gemm as OG
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+
+    # ---- headline: FP8 a8w8 prefill ------------------------------------------------------------
+    M, N, K = 8192, 28672, 8192
+    aq, wq, sa, sw = fp8_inputs(M, N, K, dev, 2)
+    b = wq.T                                   # (K, N) view of the (N, K) weight: K-contiguous
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    sel = tb.OrigamiMatmulSelector(M, N, K, aq.dtype, b.dtype, c.dtype, dev)
+    cfg = tb.matmul_preamble(sel, dev)
+    step = lambda: tb.matmul_a8w8_lt(aq, b, sa, sw, c, sel, cfg)
+    ms, wall_ms = timed(step, args.steps, args.warmup)
+    flops = 2.0 * M * N * K
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    # parity spot check on rows spread over the output (oracle on the host)
+    rows = torch.arange(0, M, 613)[:14]
+    want = OG.ref_gemm(aq[rows].cpu(), b.cpu(), torch.float32, a_scale=sa[rows].cpu(), b_scale=sw.cpu()).to(torch.bfloat16)
+    err = OG.rel_fro_error(c[rows].float().cpu(), want.float())
+
+    out = {
+        "metric": "TFLOP/s & % MFMA peak: FP8 a8w8 8192x28672x8192; MXFP4 8192x8192x16384",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3", "data": "synthetic (seeded N(0,1) bf16, per-row/per-column amax/448 scales)",
+        "config": {"workload": "FP8 a8w8 GEMM M=8192 N=28672 K=8192, bf16 out, scales in epilogue",
+                   "tile": [sel.block_m, sel.block_n, sel.block_k], "schedule": "persistent"},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_TFLOPS["fp8"], 4), "traffic": None},
+        "parity_rel_fro": float(f"{err:.3e}"),
+        "wall_ms_per_step": round(wall_ms, 4),
+        "device": {"name": props.name, "cus": props.multi_processor_count, "arch": getattr(props, "gcnArchName", "")},
+    }
+
+    # ---- CPU baseline: torch.matmul fp32 over a bounded row slice of the same problem -----------
+    if not args.skip_cpu:
+        ms_rows = 1024
+        a_s = aq[:ms_rows].cpu()
+        b_cpu = b.cpu()
+        a32, b32 = a_s.to(torch.float32), b_cpu.to(torch.float32)
+        torch.matmul(a32[:64], b32)
+        best = None
+        for _ in range(2):
+            t0 = time.perf_counter()
+            OG.ref_gemm(a_s, b_cpu, torch.float32, a_scale=sa[:ms_rows].cpu(), b_scale=sw.cpu())
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        out["cpu_baseline"] = {"value": round(2.0 * ms_rows * N * K / best / 1e12, 4), "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"rows 0..{ms_rows - 1} of the same GEMM ({ms_rows}x{N}x{K}), "
+                                         f"oracle fp32 torch.matmul of the dequantised operands + scale epilogue, best of 2, "
+                                         f"{best:.2f} s; os.cpu_count()={os.cpu_count()}"}
+        del a32, b32, b_cpu
+    del aq, wq, c, b
+
+    # ---- secondary figures ----------------------------------------------------------------------
+    if not args.skip_secondary:
+        sec = {}
+        steps2, warm2 = max(10, args.steps // 2), max(3, args.warmup // 2)
+        # MXFP4: quantise A with the fused rotate+quant kernel (timed), B rotated + quantised the same way
+        M4, N4, K4 = 8192, 8192, 16384
+        g = torch.Generator(device=dev).manual_seed(5)
+        def src(rows):
+            x = torch.randn(rows, K4, device=dev, generator=g, dtype=torch.float32)
+            mask = torch.rand(rows, K4, device=dev, generator=g) < 1e-3
+            return torch.where(mask, x * 20.0, x).bfloat16()
+        a4, b4 = src(M4), src(N4)
+        qms, _ = timed(lambda: U.hadamard_mxfp4_quant(a4), steps2, warm2)
+        qbytes = M4 * K4 * 2 + M4 * K4 // 2 + M4 * K4 // 32
+        sec["hadamard_mxfp4_quant_8192x16384"] = {"ms": round(qms, 4), "GB/s": round(qbytes / qms / 1e6, 1),
+                                                  "frac_hbm_peak": round(qbytes / qms / 1e6 / PEAK_HBM_GBPS, 4),
+                                                  "note": "includes the two output allocations of the Python wrapper"}
+        aq4, as4 = U.hadamard_mxfp4_quant(a4)
+        bq4, bs4 = U.hadamard_mxfp4_quant(b4)
+        del a4, b4
+        c4 = torch.empty(M4, N4, dtype=torch.bfloat16, device=dev)
+        fms, _ = timed(lambda: tb.matmul_fp4(aq4, bq4, c4, as4, bs4), steps2, warm2)
+        tf4 = 2.0 * M4 * N4 * K4 / fms / 1e9
+        sec["mxfp4_gemm_8192x8192x16384"] = {"ms": round(fms, 4), "TFLOP/s": round(tf4, 1),
+                                             "frac_mfma_peak": round(tf4 / PEAK_TFLOPS["mxfp4"], 4)}
+        del aq4, bq4, c4
+        # bf16 TN 8192^3
+        a2 = (torch.rand(8192, 8192, device=dev, generator=g) * 2 - 1).bfloat16()
+        b2 = (torch.rand(8192, 8192, device=dev, generator=g) * 2 - 1).bfloat16().T
+        c2 = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
+        sel2 = tb.OrigamiMatmulSelector(8192, 8192, 8192, a2.dtype, b2.dtype, c2.dtype, dev)
+        bms, _ = timed(lambda: tb.matmul_lt(a2, b2, c2, sel2, None), steps2, warm2)
+        tf2 = 2.0 * 8192 ** 3 / bms / 1e9
+        sec["bf16_gemm_8192x8192x8192_TN"] = {"ms": round(bms, 4), "TFLOP/s": round(tf2, 1),
+                                              "frac_mfma_peak": round(tf2 / PEAK_TFLOPS["bf16"], 4)}
+        del a2, b2, c2
+        # FP8 decode, Stream-K
+        Md, Nd, Kd = 32, 8192, 28672
+        aqd, wqd, sad, swd = fp8_inputs(Md, Nd, Kd, dev, 22)
+        cd = torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev)
+        seld = tb.OrigamiMatmulSelector(Md, Nd, Kd, aqd.dtype, wqd.dtype, cd.dtype, dev, streamk=True)
+        cfgd = tb.matmul_preamble(seld, dev)
+        dms, _ = timed(lambda: tb.matmul_a8w8_lt(aqd, wqd.T, sad, swd, cd, seld, cfgd, enable_streamk=True), steps2 * 4, warm2)
+        dbytes = Md * Kd + Nd * Kd + Md * Nd * 2 + (Md + Nd) * 4
+        sec["fp8_decode_32x8192x28672_streamk"] = {"ms": round(dms, 4), "GB/s": round(dbytes / dms / 1e6, 1),
+                                                   "frac_hbm_peak": round(dbytes / dms / 1e6 / PEAK_HBM_GBPS, 4),
+                                                   "tile": [seld.block_m, seld.block_n, seld.block_k], "grid": seld.sk_grid}
+        del aqd, wqd, cd
+        # grouped MoE FP8
+        E, Ng, Kg, T = 8, 14336, 4096, 4096
+        idx = torch.multinomial(torch.ones(T, E), 2, replacement=False, generator=torch.Generator().manual_seed(3))
+        counts = torch.bincount(idx.flatten(), minlength=E)
+        offs = torch.zeros(E + 1, dtype=torch.int32)
+        offs[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        ag = torch.randn(2 * T, Kg, device=dev, generator=g).bfloat16()
+        wg = torch.randn(E, Ng, Kg, device=dev, generator=g).bfloat16()
+        agq, sag = U.quantize_tensor_per_channel(ag, torch.float8_e4m3fn, axis=1)
+        wgq, swg = U.quantize_tensor_per_channel(wg, torch.float8_e4m3fn, axis=2)
+        del ag, wg
+        cg = torch.empty(2 * T, Ng, dtype=torch.bfloat16, device=dev)
+        offs_d = offs.to(dev)
+        gms, _ = timed(lambda: tb.grouped_matmul_a8w8(agq, wgq, sag, swg, cg, offs_d), steps2, warm2)
+        tfg = 2.0 * 2 * T * Ng * Kg / gms / 1e9
+        sec["grouped_moe_fp8_8x[rows x 4096]x[4096 x 14336]"] = {"ms": round(gms, 4), "TFLOP/s": round(tfg, 1),
+                                                                 "frac_mfma_peak": round(tfg / PEAK_TFLOPS["fp8"], 4)}
+        out["secondary"] = sec
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

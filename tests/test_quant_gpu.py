@@ -53,7 +53,8 @@ def test_every_bf16_bit_pattern(hadamard):
         rows.append(torch.cat([blk, col], dim=1))
     x = torch.cat(rows, dim=0)
     if hadamard:
-        x = torch.where(torch.isinf(x), torch.zeros_like(x), x)   # inf - inf inside the rotation is NaN: unspecified
+        # sums of 32 huge values overflow and inf - inf inside the rotation is NaN: unspecified
+        x = torch.where(x.float().abs() > 1e36, torch.zeros_like(x), x)
     _assert_same(x, hadamard)
 
 
