@@ -48,6 +48,7 @@ struct GemmParams {
   int32_t tiles_m, tiles_n, total_tiles, k_iters;
   int32_t group_m, num_xcds, chunk;
   int32_t mode;
+  int32_t debug;                 // tuning experiments: bit0 skip global->LDS copies, bit1 skip MFMA work
   // Stream-K
   int32_t sk_tiles;
   float* P;
@@ -72,7 +73,7 @@ struct TileCtx {
 };
 
 template <int DT_, int BM_, int BN_, int BKB_, int WM_, int WN_, int ALAY_, int BLAY_, int MINB_ = 1,
-          bool FAST_ = true, int STAGES_ = 2>
+          bool FAST_ = true, int STAGES_ = 2, bool USE_DMA_ = true>
 struct Tile {
   static constexpr int DT = DT_, BM = BM_, BN = BN_, BKB = BKB_, WM = WM_, WN = WN_;
   static constexpr int ALAY = ALAY_, BLAY = BLAY_, MINB = MINB_, STAGES = STAGES_;
@@ -80,7 +81,7 @@ struct Tile {
   // of the K step (and row counts of M-contiguous operands multiples of 8): loaders carry no
   // bounds handling besides clamping rows.  !FAST: element-wise gathers, any strides, any K.
   static constexpr bool FAST = FAST_;
-  static constexpr bool DMA = FAST && ALAY == LAY_K && BLAY == LAY_K;  // global -> LDS without registers
+  static constexpr bool DMA = USE_DMA_ && FAST && ALAY == LAY_K && BLAY == LAY_K;  // global -> LDS without registers
   static constexpr int THREADS = WM * WN * 64;
   static constexpr int USZ = (DT == DT_F16 || DT == DT_BF16) ? 2 : 1;  // bytes per storage unit
   static constexpr int UPC = 16 / USZ;                                 // units per 16-byte chunk
@@ -95,15 +96,17 @@ struct Tile {
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-  // XOR swizzle of the chunk index so that 16 rows read at one k hit 16 different bank groups.
-  static constexpr int RPL = (CPR >= 16) ? 1 : 16 / CPR;   // tile rows per 256-byte LDS line
-  static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // swizzle period
+  static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // XOR-swizzle range of the chunk index
   static_assert(CPR % KS == 0, "K step must hold whole MFMA slices");
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be MFMA aligned");
   static_assert(DT != DT_FP4 || KSUB == 1 || KSUB == 2 || KSUB == 4, "fp4 scale packing");
-  static_assert(STAGES == 2 || (DMA && STAGES == 3), "deeper pipelines need the LDS-direct loader");
+  static_assert(STAGES == 2 || (DMA && STAGES <= 4), "deeper pipelines need the LDS-direct loader");
   static_assert((BM * CPR) % 64 == 0 && (BN * CPR) % 64 == 0, "whole waves per operand copy");
-  __device__ static __forceinline__ int swz(int row) { return (row / RPL) % SWM; }
+  // XOR mask applied to the chunk index of a row: the low row bits, with odd and even groups of SWM
+  // rows offset by one so that the 16 rows one MFMA operand read touches spread over all banks.
+  __device__ static __forceinline__ int swz(int row) {
+    return (SWM < 16) ? (((row % SWM) ^ ((row / SWM) & 1)) % SWM) : (row % SWM);
+  }
 };
 
 struct LaneInfo {
@@ -213,16 +216,23 @@ struct Operand {
     else return st.base + (int64_t)it * T::UPS * st.s_k * 2;
   }
 
-  // LDS-direct copy of K step `it` into `lds` (no registers involved)
+  // LDS-direct copy of K step `it` into `lds` (no registers involved).  Written as inline assembly
+  // for two reasons: the address is a scalar base plus a loop-invariant 32-bit lane offset, and the
+  // compiler must not know that these vector-memory operations write LDS, otherwise it drains every
+  // outstanding copy (vmcnt(0)) in front of the next LDS read and the software pipeline collapses.
+  // Completion is tracked by hand with s_waitcnt vmcnt(N) before the barrier that publishes a stage.
   __device__ static __forceinline__ void dma(const St& st, int it, uint8_t* lds, int tid) {
     const uint8_t* gp = step_ptr(st, it);
     const int wave_slot = __builtin_amdgcn_readfirstlane(tid & ~63);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       if (CHUNKS % T::THREADS != 0 && i * T::THREADS + wave_slot >= CHUNKS) continue;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gp + st.off[i]),
-                                       (__attribute__((address_space(3))) void*)(lds + (i * T::THREADS + wave_slot) * 16),
-                                       16, 0, 0);
+      const uint32_t dst = lds0 + (uint32_t)((i * T::THREADS + wave_slot) * 16);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(dst), "v"(st.off[i]), "s"(gp)
+                   : "memory", "m0");
     }
   }
 
@@ -400,31 +410,50 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     }
   };
 
+  // One K step of MFMAs from an LDS stage.  The A-side fragment of row block i+1 is requested before
+  // the MFMAs of row block i are issued, so an LDS read is always in flight under the matrix pipe.
   auto compute = [&](const uint8_t* sA, const uint8_t* sB) {
 #pragma unroll
     for (int ks = 0; ks < T::KSUB; ++ks) {
       frag_t bf[T::TN];
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) bf[j] = Frag<T>::read(sB, li.wn0 + j * 16 + li.r, ks, li.g, swm);
+      frag_t af[2];
+      af[0] = Frag<T>::read(sA, li.wm0 + li.r, ks, li.g, swm);
 #pragma unroll
       for (int i = 0; i < T::TM; ++i) {
-        frag_t af = Frag<T>::read(sA, li.wm0 + i * 16 + li.r, ks, li.g, swm);
+        if (i + 1 < T::TM) af[(i + 1) & 1] = Frag<T>::read(sA, li.wm0 + (i + 1) * 16 + li.r, ks, li.g, swm);
 #pragma unroll
         for (int j = 0; j < T::TN; ++j) {
           // output rows follow the first MFMA operand: feed B there so that one lane owns four
           // consecutive n of one m (contiguous in a row-major C).
-          if (ks == 0) acc[i][j] = mma<T, 0>(bf[j], af, acc[i][j], scb[j], sca[i]);
-          if (ks == 1) acc[i][j] = mma<T, 1>(bf[j], af, acc[i][j], scb[j], sca[i]);
-          if (ks == 2) acc[i][j] = mma<T, 2>(bf[j], af, acc[i][j], scb[j], sca[i]);
-          if (ks == 3) acc[i][j] = mma<T, 3>(bf[j], af, acc[i][j], scb[j], sca[i]);
+          if (ks == 0) acc[i][j] = mma<T, 0>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
+          if (ks == 1) acc[i][j] = mma<T, 1>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
+          if (ks == 2) acc[i][j] = mma<T, 2>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
+          if (ks == 3) acc[i][j] = mma<T, 3>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
         }
       }
+      // pin the issue order for the machine scheduler: B fragments and the first A fragment, then
+      // alternately the next A fragment's reads and one row block of MFMAs
+      constexpr int RPF = (T::DT == DT_FP8) ? 2 : 1;  // LDS reads per fragment
+      __builtin_amdgcn_sched_group_barrier(0x100, RPF * (T::TN + 1), 0);
+#pragma unroll
+      for (int i = 0; i + 1 < T::TM; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, T::TN, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, T::TN, 0);
     }
   };
 
   if constexpr (T::DMA) {
     constexpr int S = T::STAGES;
-    // stage s of iteration it: lds + ((it - it0) % S) * STAGE_BYTES; copies run S-1 iterations ahead.
+    // Stage (it - it0) % S holds K step `it`; copies run S-1 steps ahead of the MFMAs.  One "group" is
+    // what a wave issues per K step: its share of both operand copies, then (fp4) its scale loads.
+    constexpr int NI = OA::NCH + OB::NCH;
+    constexpr int NSC = (T::DT == DT_FP4) ? (T::TM + T::TN) : 0;
+    constexpr int NG = NI + NSC;
+    static_assert((S - 2) * NG + NSC <= 63, "vmcnt range");
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) {
       if (it0 + s < it1) {
@@ -433,29 +462,29 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
     }
     load_scales(it0, sca, scb);
-    if (S == 3 && it0 + 1 < it1) __builtin_amdgcn_s_waitcnt(0x0F70 | 0);  // conservative: everything landed
-    else wait_vm0();
+    wait_vm0();
     __syncthreads();
     int stage = 0;
     for (int it = it0; it < it1; ++it) {
       const int nxt = it + S - 1;
       int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
-      if (nxt < it1) {
+      if (nxt < it1 && !(p.debug & 1)) {
         OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
         OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
       if (it + 1 < it1) load_scales(it + 1, nsca, nscb);
-      compute(lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      if (!(p.debug & 2)) compute(lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
       if (it + 1 < it1) {
 #pragma unroll
         for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
 #pragma unroll
         for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j];
       }
-      // the next iteration's stage must have landed; with three stages one copy group may stay in flight
-      if (S == 3 && T::DT != DT_FP4 && nxt < it1) {
-        constexpr int NI = OA::NCH + OB::NCH;
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (NI & 0xF) | ((NI >> 4) << 14));
+      // K step it+1 must have landed before the barrier; the S-2 younger groups may stay in flight.
+      // (vmcnt counts in issue order; near the end of the tile fewer groups exist, so drain fully.)
+      if (S > 2 && nxt < it1) {
+        constexpr int ALLOWED = (S - 2) * NG;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
       } else {
         wait_vm0();
       }
@@ -480,7 +509,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::gload(rb, sb, it + 1, p.KU, li.tid);
         load_scales(it + 1, nsca, nscb);
       }
-      compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
+      if (!(p.debug & 2)) compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
       if (has_next) {
         OA::sstore(sA0 + (cur ^ 1) * T::STAGE_BYTES, ra, li.tid);
         OB::sstore(sB0 + (cur ^ 1) * T::STAGE_BYTES, rb, li.tid);

@@ -11,7 +11,7 @@ namespace tb {
   make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_M, LAY_M, MINB, true, 2>>()
 
 const Variant g_variants_f16[] = {
-    TB_LAYOUTS(256, 256, 2, 2, 1),
+    TB_LAYOUTS(256, 256, 2, 4, 1),
     TB_LAYOUTS(128, 128, 2, 2, 2),
     TB_LAYOUTS(64, 64, 2, 2, 4),
     make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),

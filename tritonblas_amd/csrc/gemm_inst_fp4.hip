@@ -4,7 +4,7 @@
 namespace tb {
 
 const Variant g_variants_fp4[] = {
-    make_variant<Tile<DT_FP4, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>>(),
+    make_variant<Tile<DT_FP4, 256, 256, 128, 2, 4, LAY_K, LAY_K, 1, true, 2>>(),
     make_variant<Tile<DT_FP4, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_FP4, 128, 128, 64, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_FP4, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),

@@ -5,7 +5,7 @@
 namespace tb {
 
 const Variant g_variants_fp8[] = {
-    make_variant<Tile<DT_FP8, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>>(),
+    make_variant<Tile<DT_FP8, 256, 256, 128, 2, 4, LAY_K, LAY_K, 1, true, 2>>(),
     make_variant<Tile<DT_FP8, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),
     make_variant<Tile<DT_FP8, 32, 128, 256, 1, 4, LAY_K, LAY_K, 1, true, 3>>(),

@@ -8,14 +8,14 @@ namespace tb {
 struct Variant {
   int dt, bm, bn, bk;     // element type and tile in elements
   int alay, blay;         // operand loaders (LAY_K / LAY_M)
-  int threads, lds_bytes, minb;
+  int wm, wn, threads, lds_bytes, minb;
   int fast, stages;       // fast: vector/LDS-direct loaders (alignment + K multiple required)
   const void* kernel;     // __global__ void (*)(const GemmParams)
 };
 
 template <class T>
 constexpr Variant make_variant() {
-  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::THREADS, T::LDS_BYTES + 16, T::MINB,
+  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_BYTES + 16, T::MINB,
                  T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T>};
 }
 

@@ -52,51 +52,58 @@ int variant_occupancy(const TileInfo& v, const tb_hw& hw) {
   return std::max(1, std::min({by_lds, by_waves, v.minb}));
 }
 
+// Measured behaviour of the built kernels on MI355X that the model is anchored to:
+//   * MFMA-side efficiency of the K loop with operands already in LDS (fraction of the matrix pipe):
+//     256x256 tiles ~0.47, 128x128 ~0.64, 64x64 ~0.55, the skinny 32x128 tile ~0.30;
+//   * L2 -> LDS fill rate per CU: ~16 B/clk with one workgroup per CU, ~30 B/clk with two or more
+//     (the vector L1 keeps a bounded number of lines in flight, so the rate is latency-bound).
+static double mfma_side_efficiency(const TileInfo& v) {
+  const int area = v.bm * v.bn;
+  if (area >= 256 * 256) return 0.47;
+  if (area >= 128 * 128) return 0.64;
+  if (area >= 64 * 64) return 0.55;
+  return 0.30;
+}
+
 static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk, double* comp_us,
                     double* mem_us) {
   const double clk = hw.clock_khz * 1e3;
   const int bits = type_bits(pr.a_type);
   const double esz = bits / 8.0;
   const int64_t tiles_m = cdiv(pr.m, v.bm), tiles_n = cdiv(pr.n, v.bn);
-  const int64_t tiles = tiles_m * tiles_n + (pr.num_groups > 0 ? pr.num_groups * tiles_n / 2 : 0);
+  const int64_t tiles = tiles_m * tiles_n + (pr.num_groups > 0 ? (int64_t)pr.num_groups * tiles_n / 2 : 0);
   const int64_t k_iters = cdiv(pr.k, v.bk);
   const int occ = variant_occupancy(v, hw);
-  const int waves = v.threads / 64;
   const double bkb = v.bk * esz;
 
-  // per K step, per workgroup (cycles)
-  const double t_mfma = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type);
-  const int wm = (v.bm >= v.bn) ? std::max(1, waves / 2) : 1;  // informational split, matches the built shapes
-  (void)wm;
-  const double wave_rows = (double)v.bm / 2 + (double)v.bn / 2;  // rows each of the 2x2 waves reads
-  const double t_lds = waves * wave_rows * bkb / 128.0;          // 128 B/clk/CU LDS read
-  const double t_fill = (v.bm + v.bn) * bkb / 64.0;              // L2 -> LDS, 64 B/clk/CU
-  const double t_sync = 120.0;
-  double t_iter;
-  if (occ >= 2) t_iter = std::max({t_mfma, t_lds, t_fill}) + t_sync / occ;   // workgroups overlap each other
-  else t_iter = std::max(t_mfma + 0.25 * t_lds, std::max(t_lds, t_fill)) + t_sync;
+  // per K step of one workgroup, in CU cycles (MFMA pipe and fill path are shared by the CU)
+  const double t_mfma = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type) / mfma_side_efficiency(v);
+  const double t_fill = (v.bm + v.bn) * bkb / (occ >= 2 ? 30.0 : 16.0);
+  const double t_iter = std::max(t_mfma, t_fill) + 60.0;
   const double c_bytes = type_bits(pr.c_type) / 8.0;
-  const double t_epi = 1500.0 + v.bm * v.bn * c_bytes / 32.0;
-  const double t_tile = k_iters * t_iter + t_epi;
+  const double t_epi = 2500.0 + v.bm * v.bn * c_bytes / 32.0;
 
   double cycles;
   if (streamk) {
-    // iterations spread evenly over all resident workgroups, one fixup per workgroup
+    // K iterations spread evenly over every resident workgroup slot; one partial-tile fixup each
     const double slots = (double)hw.n_cu * occ;
-    const double iters_per_wg = std::ceil((double)tiles * k_iters / slots);
-    cycles = iters_per_wg * t_iter * occ + t_epi * std::max(1.0, (double)tiles / slots) + 2000.0;
+    const double iters_per_cu = std::ceil((double)tiles * k_iters / slots) * occ;
+    cycles = iters_per_cu * t_iter + t_epi * std::max(1.0, (double)tiles / slots) + 6000.0;
   } else {
-    const double rounds = std::ceil((double)tiles / ((double)hw.n_cu * occ));
-    cycles = rounds * t_tile * occ;  // occ workgroups share the CU's MFMA/LDS throughput
-    if (occ >= 2) cycles = std::max(cycles, rounds * (k_iters * t_mfma * occ + t_epi));
+    const double rounds = std::ceil((double)tiles / (double)hw.n_cu);  // tiles one CU works through
+    cycles = rounds * (k_iters * t_iter + t_epi / occ);
+    // a partly filled last round leaves CUs idle; small grids cannot use the L2-hit fill rate either
+    if (tiles < hw.n_cu) cycles = k_iters * t_iter + t_epi;
   }
   *comp_us = cycles / clk * 1e6;
 
   // HBM: every operand once, plus re-reads when a band of tiles does not stay in L2/MALL
   const double a_bytes = (double)pr.m * pr.k * esz, b_bytes = (double)pr.n * pr.k * esz * std::max(1, pr.num_groups);
   const double c_out = (double)pr.m * pr.n * c_bytes;
-  const double reread = 1.0 + 0.15 * std::max(0.0, std::log2((double)std::max<int64_t>(1, 256 / std::min(v.bm, v.bn))));
-  *mem_us = ((a_bytes + b_bytes) * reread + c_out) / (hw.hbm_gbps * 1e9 * 0.8) * 1e6;
+  // few workgroups cannot pull the full HBM rate: ~45 GB/s per busy CU
+  const double busy_cus = std::min<double>(hw.n_cu, streamk ? hw.n_cu : (double)tiles);
+  const double hbm = std::min(hw.hbm_gbps * 0.65, busy_cus * 45.0);
+  *mem_us = (a_bytes + b_bytes + c_out) / (hbm * 1e9) * 1e6;
   return std::max(*comp_us, *mem_us) + 3.0;
 }
 
@@ -107,6 +114,11 @@ int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, in
     const TileInfo& v = tiles[i];
     if (!v.fast) continue;  // the gather kernels are a fallback, never a choice of the model
     if (v.lds_bytes > hw.lds_bytes) continue;
+    // decode-like problems (a handful of rows): tiles taller than twice the row count only add
+    // LDS traffic and idle MFMA rows when a shorter tile exists
+    bool shorter_exists = false;
+    for (int q = 0; q < ntiles; ++q) shorter_exists |= tiles[q].fast && tiles[q].bm < v.bm && tiles[q].bm >= pr.m;
+    if (shorter_exists && pr.num_groups == 0) continue;
     double c, m;
     double t = score(pr, hw, v, pr.streamk != 0, &c, &m);
     // prefer the larger tile on ties (less L2 traffic than the model resolves)

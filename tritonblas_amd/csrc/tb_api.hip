@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -89,6 +90,14 @@ std::vector<TileInfo> tile_infos(int dt) {
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
+  // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
+  const char* wenv = getenv("TB_WAVES");
+  const int want = wenv ? atoi(wenv) : 0;
+  if (want && fast)
+    for (int i = 0; i < n; ++i)
+      if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
+          (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want))
+        return &v[i];
   for (int i = 0; i < n; ++i)
     if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk)))
       return &v[i];
@@ -222,6 +231,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.group_m = j.group_m > 0 ? j.group_m : std::min(8, (int)p.tiles_m);
   p.num_xcds = j.num_xcds > 0 ? j.num_xcds : hw.num_xcd;
   p.epoch = j.epoch; p.spin_limit = j.spin_limit ? j.spin_limit : (1u << 24);
+  { const char* dbg = getenv("TB_DEBUG"); p.debug = dbg ? atoi(dbg) : 0; }
   p.group_offsets = j.group_offsets; p.num_groups = j.num_groups;
   p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
 
