@@ -39,6 +39,17 @@ def timed(fn, steps, warmup):
     return start.elapsed_time(end) / steps, wall_ms
 
 
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size); None when no summary is present."""
+    path = os.path.join(ROOT, "profiles", "fp8_gemm_8192x28672x8192_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f)["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def fp8_inputs(m, n, k, dev, seed):
     import tritonblas_amd.utils as U
     g = torch.Generator(device=dev).manual_seed(seed)
@@ -57,6 +68,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-secondary", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known HBM bytes) so that FETCH_SIZE / WRITE_SIZE "
+                         "readings of a rocprofv3 --pmc run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1", file=sys.stderr)
@@ -68,6 +82,14 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     props = torch.cuda.get_device_properties(dev)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- headline: FP8 a8w8 prefill ------------------------------------------------------------
     M, N, K = 8192, 28672, 8192
@@ -94,7 +116,7 @@ def main():
         "config": {"workload": "FP8 a8w8 GEMM M=8192 N=28672 K=8192, bf16 out, scales in epilogue",
                    "tile": [sel.block_m, sel.block_n, sel.block_k], "schedule": "persistent"},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_TFLOPS["fp8"], 4), "traffic": None},
+                     "frac": round(tflops / PEAK_TFLOPS["fp8"], 4), "traffic": measured_traffic()},
         "parity_rel_fro": float(f"{err:.3e}"),
         "wall_ms_per_step": round(wall_ms, 4),
         "device": {"name": props.name, "cus": props.multi_processor_count, "arch": getattr(props, "gcnArchName", "")},

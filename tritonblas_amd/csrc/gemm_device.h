@@ -668,7 +668,7 @@ __device__ __forceinline__ bool grouped_tile(const GemmParams& p, int tile, int 
   return false;
 }
 
-template <class T>
+template <class T, bool SK>
 struct Sched {
   int pid, G;
   int next_tile;          // static / Stream-K data-parallel phase
@@ -733,6 +733,7 @@ struct Sched {
       }
       return false;
     }
+    if constexpr (!SK) return false;
     // MODE_SK: data-parallel tiles first, then this workgroup's share of the Stream-K iterations
     if (next_tile < dp_tiles) {
       plain_tile(p, next_tile, T::BM, T::BN, w.tc);
@@ -755,7 +756,10 @@ struct Sched {
   }
 };
 
-template <class T>
+// SK = false: data-parallel, work-stealing and grouped schedules (every work item is a whole tile).
+// SK = true: adds the Stream-K tail with its partial-tile publish / fixup paths.  Two kernels, so that
+// the accumulator-heavy fixup code cannot push the common path into register spills.
+template <class T, bool SK>
 __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_BYTES];
   __shared__ int s_bcast;
@@ -769,12 +773,13 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   li.wn0 = (wave % T::WN) * T::WTN;
   v4f acc[T::TM][T::TN];
 
-  Sched<T> sched;
+  Sched<T, SK> sched;
   sched.init(p);
   Work w;
   bool failed = false;
   while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
     mainloop<T>(p, w.tc, w.it0, w.it1, acc, lds, li);
+    if constexpr (SK) {
     if (w.kind == WK_SK_PUBLISH) {
       // not the tile's first segment: publish the partial, tagged with this launch's epoch
       partial_store<T>(p.P + (size_t)sched.pid * (T::BM * T::BN), acc, li.tid);
@@ -808,10 +813,13 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
       }
       if (failed) break;
     }
+    }
     epilogue<T>(p, w.tc, acc, li);
   }
-  if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
-  if (p.mode == MODE_WS && li.tid == 0) {
+  if constexpr (SK) {
+    if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
+  }
+  if (!SK && p.mode == MODE_WS && li.tid == 0) {
     // the last workgroup to leave rearms the queues for the next launch
     uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
     if (done == gridDim.x - 1) {

@@ -135,14 +135,14 @@ struct Plan {
   size_t ws_need = 0, ws_flags_off = 0, ws_p_off = 0, ws_counters_off = 0;
 };
 
-int kernel_occupancy(const Variant* v) {
+int kernel_occupancy(const Variant* v, const void* kernel) {
   static std::mutex mu;
   static std::vector<std::pair<const void*, int>> cache;
   std::lock_guard<std::mutex> lk(mu);
-  for (auto& c : cache) if (c.first == v->kernel) return c.second;
+  for (auto& c : cache) if (c.first == kernel) return c.second;
   int nb = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->kernel, v->threads, 0) != hipSuccess || nb < 1) nb = 1;
-  cache.emplace_back(v->kernel, nb);
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel, v->threads, 0) != hipSuccess || nb < 1) nb = 1;
+  cache.emplace_back(kernel, nb);
   return nb;
 }
 
@@ -235,7 +235,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.group_offsets = j.group_offsets; p.num_groups = j.num_groups;
   p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
 
-  const int occ = need_device ? kernel_occupancy(v) : std::max(1, std::min(v->minb, hw.lds_bytes / v->lds_bytes));
+  const void* kern = (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) ? v->kernel_sk : v->kernel;
+  const int occ = need_device ? kernel_occupancy(v, kern) : std::max(1, std::min(v->minb, hw.lds_bytes / v->lds_bytes));
   const int resident = hw.n_cu * occ;
   int grid;
   plan->ws_need = 0;
@@ -286,7 +287,8 @@ int launch(const Job& j, hipStream_t stream) {
     if (p.mode == MODE_SK) { p.flags = (uint32_t*)(ws + plan.ws_flags_off); p.P = (float*)(ws + plan.ws_p_off); }
   }
   void* args[] = {(void*)&p};
-  hipError_t e = hipLaunchKernel(plan.v->kernel, dim3((unsigned)plan.grid), dim3((unsigned)plan.v->threads), args, 0, stream);
+  const void* kern = (p.mode == MODE_SK) ? plan.v->kernel_sk : plan.v->kernel;
+  hipError_t e = hipLaunchKernel(kern, dim3((unsigned)plan.grid), dim3((unsigned)plan.v->threads), args, 0, stream);
   if (e != hipSuccess) { (void)hipGetLastError(); return TB_ERR_LAUNCH; }
   return TB_OK;
 }
