@@ -43,7 +43,8 @@ struct GemmParams {
   int64_t mxa_sr, mxa_sk, mxb_sr, mxb_sk;  // bytes
   int64_t bias_stride;
   int32_t c_type, bias_type;
-  int32_t a_vec, b_vec, c_vec;   // 16-byte vector access is legal for this operand
+  int32_t a_vec, b_vec, c_vec;   // 16-byte vector access is legal for this operand (c_vec: 4-element rows)
+  int32_t c_line;                // C rows are 16-byte aligned with unit column stride: full-line store path
   int32_t mx_vec;                // scale rows can be read KSUB bytes at a time
   int32_t tiles_m, tiles_n, total_tiles, k_iters;
   int32_t group_m, num_xcds, chunk;
@@ -599,9 +600,115 @@ __device__ __forceinline__ void epilogue_t(const GemmParams& p, const TileCtx& t
   }
 }
 
+// Full-line variant for a row-major C with 16-byte aligned rows: every wave transposes its own
+// accumulator tile through a private LDS region (rows padded by 16 bytes so that the 8-byte writes
+// of the 16 rows x 4 lane groups spread over the banks), then writes 16 bytes per lane, 8 lanes per
+// 128-byte row segment.  No barrier is involved: a wave only reads what it wrote itself.
+template <class T, int CT>
+__device__ __forceinline__ void epilogue_lines(const GemmParams& p, const TileCtx& tc, v4f (&acc)[T::TM][T::TN],
+                                               const LaneInfo& li, uint8_t* lds) {
+  constexpr int CS = (CT == DT_F32) ? 4 : 2;
+  constexpr int ROWB = T::WTN * CS;            // bytes of one wave-tile row
+  constexpr int RS = ROWB + 16;                // padded LDS row stride
+  constexpr int WAVES = T::WM * T::WN;
+  constexpr int MAXROWS = (T::LDS_BYTES / WAVES / RS) / 16 * 16;
+  constexpr int PASS_TM = (MAXROWS / 16 >= T::TM) ? T::TM : MAXROWS / 16;   // row blocks per pass
+  static_assert(PASS_TM >= 1, "LDS too small for the store staging");
+  constexpr int CPRW = ROWB / 16;              // 16-byte chunks per row
+  constexpr int ROWS_PER_INST = 64 / CPRW;
+  uint8_t* stage = lds + (li.tid >> 6) * (PASS_TM * 16 * RS);
+
+  float sav[T::TM];
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i) {
+    int m = tc.m0 + li.wm0 + i * 16 + li.r;
+    sav[i] = (p.sa && m < tc.m_lim) ? p.sa[m] : 1.f;
+  }
+  v4f sbv[T::TN], bv[T::TN];
+#pragma unroll
+  for (int j = 0; j < T::TN; ++j) {
+    int n = tc.n0 + li.wn0 + j * 16 + 4 * li.g;
+    int nvalid = tc.n_lim - n;
+    sbv[j] = v4f{1.f, 1.f, 1.f, 1.f};
+    bv[j] = v4f{0.f, 0.f, 0.f, 0.f};
+    if (tc.sb) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) if (q < nvalid) sbv[j][q] = tc.sb[n + q];
+    }
+    if (p.bias) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (q < nvalid) bv[j][q] = load_as_f32(p.bias + (int64_t)(n + q) * p.bias_stride * (p.bias_type == DT_F32 ? 4 : 2), p.bias_type);
+    }
+  }
+#pragma unroll
+  for (int i0 = 0; i0 < T::TM; i0 += PASS_TM) {
+#pragma unroll
+    for (int ii = 0; ii < PASS_TM; ++ii) {
+      const int i = i0 + ii;
+      if (i >= T::TM) continue;
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+        v4f v = acc[i][j];
+        if (p.sa) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = v[q] * (sav[i] * sbv[j][q]);
+        }
+        if (p.bias) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = v[q] + bv[j][q];
+        }
+        uint8_t* dst = stage + (ii * 16 + li.r) * RS + (j * 16 + 4 * li.g) * CS;
+        if constexpr (CT == DT_F32) {
+          *(v4f*)dst = v;
+        } else {
+          uint16_t h[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if constexpr (CT == DT_F16) h[q] = __builtin_bit_cast(uint16_t, (_Float16)v[q]);
+            else h[q] = __builtin_bit_cast(uint16_t, (__bf16)v[q]);
+          }
+          uint2 pk = {(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+          *(uint2*)dst = pk;
+        }
+      }
+    }
+    // read back row-contiguous and store full lines
+    constexpr int PROWS = PASS_TM * 16;
+#pragma unroll
+    for (int rb = 0; rb < PROWS; rb += ROWS_PER_INST) {
+      const int row = rb + li.lane / CPRW;
+      const int ch = li.lane % CPRW;
+      const int m = tc.m0 + li.wm0 + i0 * 16 + row;
+      const int n = tc.n0 + li.wn0 + ch * (16 / CS);
+      if (i0 * 16 + row >= T::WTM || m >= tc.m_lim || n >= tc.n_lim) continue;
+      const v4i val = *(const v4i*)(stage + row * RS + ch * 16);
+      uint8_t* gp = p.C + ((int64_t)m * p.c_sm + n) * CS;
+      if (n + 16 / CS <= tc.n_lim) {
+        *(v4i*)gp = val;
+      } else {
+        const uint32_t w[4] = {(uint32_t)val.x, (uint32_t)val.y, (uint32_t)val.z, (uint32_t)val.w};
+#pragma unroll
+        for (int e = 0; e < 16 / CS; ++e) {
+          if (n + e < tc.n_lim) {
+            if constexpr (CS == 4) ((uint32_t*)gp)[e] = w[e];
+            else ((uint16_t*)gp)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+          }
+        }
+      }
+    }
+  }
+}
+
 template <class T>
 __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc, v4f (&acc)[T::TM][T::TN],
-                                         const LaneInfo& li) {
+                                         const LaneInfo& li, uint8_t* lds) {
+  if (p.c_line) {
+    if (p.c_type == DT_BF16) epilogue_lines<T, DT_BF16>(p, tc, acc, li, lds);
+    else if (p.c_type == DT_F16) epilogue_lines<T, DT_F16>(p, tc, acc, li, lds);
+    else epilogue_lines<T, DT_F32>(p, tc, acc, li, lds);
+    return;
+  }
   if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);
   else if (p.c_type == DT_F16) epilogue_t<T, DT_F16>(p, tc, acc, li);
   else epilogue_t<T, DT_F32>(p, tc, acc, li);
@@ -778,6 +885,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   Work w;
   bool failed = false;
   while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
+    __syncthreads();  // the previous item's store staging may still be read by slower waves
     mainloop<T>(p, w.tc, w.it0, w.it1, acc, lds, li);
     if constexpr (SK) {
     if (w.kind == WK_SK_PUBLISH) {
@@ -814,7 +922,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
       if (failed) break;
     }
     }
-    epilogue<T>(p, w.tc, acc, li);
+    epilogue<T>(p, w.tc, acc, li, lds);
   }
   if constexpr (SK) {
     if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
