@@ -46,6 +46,7 @@ struct GemmParams {
   int32_t a_vec, b_vec, c_vec;   // 16-byte vector access is legal for this operand (c_vec: 4-element rows)
   int32_t c_line;                // C rows are 16-byte aligned with unit column stride: full-line store path
   int32_t mx_vec;                // scale rows can be read KSUB bytes at a time
+  int32_t mx_lds;                // scale rows are 16-byte aligned and K/32 is a multiple of 32: stage scales in LDS
   int32_t tiles_m, tiles_n, total_tiles, k_iters;
   int32_t group_m, num_xcds, chunk;
   int32_t mode;
@@ -97,6 +98,12 @@ struct Tile {
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  // MX scales (fp4, LDS-direct kernels): 32 scale bytes per tile row are staged in LDS at a time,
+  // i.e. the scales of SCG consecutive K steps (one 32-element block = one 16-byte chunk = one byte).
+  static constexpr int SC_GB = 32;
+  static constexpr int SCG = (DT == DT_FP4) ? SC_GB / CPR : 1;
+  static constexpr int SC_BYTES = (DT == DT_FP4 && DMA) ? (BM + BN) * SC_GB : 0;
+  static constexpr int LDS_TOTAL = LDS_BYTES + SC_BYTES;
   static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // XOR-swizzle range of the chunk index
   static_assert(CPR % KS == 0, "K step must hold whole MFMA slices");
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be MFMA aligned");
@@ -462,20 +469,94 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
     }
-    load_scales(it0, sca, scb);
+    // ---- MX scales through LDS (fp4): one group = the scale bytes of SCG K steps for every tile row ----
+    constexpr bool MXL = (T::DT == DT_FP4);
+    constexpr bool mx_lds = MXL;   // the fast fp4 kernels are only launched when the scale rows qualify
+    uint8_t* sc_lds = lds + T::LDS_BYTES;
+    constexpr int NQ = (T::BM + T::BN) * (T::SC_GB / 16);          // 16-byte scale chunks per group
+    constexpr int NSCH = MXL ? (NQ + T::THREADS - 1) / T::THREADS : 1;
+    const uint8_t* scp[NSCH];
+    uint32_t ga[T::TM][2], gb[T::TN][2];
+    int reg_group = -1, lds_group = -1, read_it = -1;
+    if constexpr (MXL) {
+#pragma unroll
+      for (int i = 0; i < NSCH; ++i) {
+        const int q = i * T::THREADS + li.tid;
+        const int row = q / (T::SC_GB / 16), part = q % (T::SC_GB / 16);
+        if (row < T::BM) scp[i] = p.mxa + (int64_t)min(tc.m0 + row, tc.m_lim - 1) * p.mxa_sr + part * 16;
+        else scp[i] = p.mxb + (int64_t)min(tc.n0 + row - T::BM, tc.n_lim - 1) * p.mxb_sr + part * 16;
+      }
+    }
+    auto sc_dma = [&](int grp) {
+      if constexpr (MXL) {
+        const int wave_slot = __builtin_amdgcn_readfirstlane(li.tid & ~63);
+        const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)sc_lds);
+#pragma unroll
+        for (int i = 0; i < NSCH; ++i) {
+          if (NQ % T::THREADS != 0 && i * T::THREADS + wave_slot >= NQ) continue;
+          const uint32_t dst = lds0 + (uint32_t)((i * T::THREADS + wave_slot) * 16);
+          const uint8_t* src = scp[i] + (int64_t)grp * T::SC_GB;
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+        }
+      }
+    };
+    auto sc_read = [&]() {
+      if constexpr (MXL) {
+        auto rd = [&](int row, uint32_t(&out)[2]) {
+          const uint8_t* b = sc_lds + row * T::SC_GB + li.g * T::KSUB;
+          out[0] = out[1] = 0;
+#pragma unroll
+          for (int s = 0; s < T::SCG; ++s) {
+            uint32_t v = (T::KSUB == 2) ? (uint32_t)(*(const uint16_t*)(b + s * T::CPR)) : (uint32_t)(*(b + s * T::CPR));
+            out[(s * T::KSUB) >> 2] |= v << (8 * ((s * T::KSUB) & 3));
+          }
+        };
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) rd(li.wm0 + i * 16 + li.r, ga[i]);
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) rd(T::BM + li.wn0 + j * 16 + li.r, gb[j]);
+      }
+    };
+    static_assert(!MXL || T::KSUB <= 2, "LDS-staged scales hold 8 bytes per lane and row block");
+
+    if (mx_lds) { sc_dma(it0 / T::SCG); lds_group = it0 / T::SCG; }
+    else load_scales(it0, sca, scb);
     wait_vm0();
     __syncthreads();
     int stage = 0;
     for (int it = it0; it < it1; ++it) {
       const int nxt = it + S - 1;
       int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
+      if (mx_lds) {
+        const int grp = it / T::SCG;
+        if (grp != reg_group) {
+          if (lds_group != grp) {  // only right after a segment start: nobody could prefetch this group
+            sc_dma(grp);
+            wait_vm0();
+            __syncthreads();
+            lds_group = grp;
+          }
+          sc_read();
+          reg_group = grp;
+          read_it = it;
+        } else if (it > read_it && lds_group == grp && (grp + 1) * T::SCG < it1) {
+          sc_dma(grp + 1);       // every wave has consumed group grp (a barrier has passed since)
+          lds_group = grp + 1;
+        }
+        const int sidx = (it % T::SCG) * T::KSUB;
+        const int sh = 8 * (sidx & 3);
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
+      }
       if (nxt < it1 && !(p.debug & 1)) {
         OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
         OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
-      if (it + 1 < it1) load_scales(it + 1, nsca, nscb);
+      if (!mx_lds && it + 1 < it1) load_scales(it + 1, nsca, nscb);
       if (!(p.debug & 2)) compute(lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
-      if (it + 1 < it1) {
+      if (!mx_lds && it + 1 < it1) {
 #pragma unroll
         for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
 #pragma unroll
@@ -483,7 +564,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
       // K step it+1 must have landed before the barrier; the S-2 younger groups may stay in flight.
       // (vmcnt counts in issue order; near the end of the tile fewer groups exist, so drain fully.)
-      if (S > 2 && nxt < it1) {
+      if (S > 2 && nxt < it1 && !MXL) {
         constexpr int ALLOWED = (S - 2) * NG;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
       } else {
@@ -868,7 +949,7 @@ struct Sched {
 // the accumulator-heavy fixup code cannot push the common path into register spills.
 template <class T, bool SK>
 __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmParams p) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_BYTES];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_TOTAL];
   __shared__ int s_bcast;
   LaneInfo li;
   li.tid = threadIdx.x;

@@ -16,7 +16,7 @@ struct Variant {
 
 template <class T>
 constexpr Variant make_variant() {
-  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_BYTES + 16, T::MINB,
+  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_TOTAL + 16, T::MINB,
                  T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>};
 }
 

@@ -183,6 +183,13 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   }
   const Variant* v = nullptr;
   bool fast = alay >= 0 && blay >= 0 && (KU % (bk / epu) == 0);
+  if (j.dt == TB_FP4_E2M1) {
+    // the fast fp4 kernels stage 32 scale bytes per row at a time through LDS with 16-byte copies
+    const bool mx_ok = j.mxa_sk == 1 && j.mxb_sk == 1 && (j.K / 32) % 32 == 0 && j.mxa_sr % 16 == 0 && j.mxb_sr % 16 == 0 &&
+                       ((uintptr_t)j.mxa % 16) == 0 && ((uintptr_t)j.mxb % 16) == 0;
+    const char* e = getenv("TB_NO_MXLDS");
+    if (!mx_ok || (e && atoi(e))) fast = false;
+  }
   if (fast) {
     // 32-bit offsets inside a tile
     if ((alay == LAY_K && (int64_t)bm * j.a_sr * usz >= (1ll << 31)) || (blay == LAY_K && (int64_t)bn * j.b_sr * usz >= (1ll << 31)) ||
@@ -223,6 +230,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     const int ksub = v->bk / 128;
     p.mx_vec = (j.mxa_sk == 1 && j.mxb_sk == 1 && j.mxa_sr % ksub == 0 && j.mxb_sr % ksub == 0 &&
                 ((uintptr_t)j.mxa % ksub) == 0 && ((uintptr_t)j.mxb % ksub) == 0) ? 1 : 0;
+    p.mx_lds = v->fast;
   }
   p.tiles_m = (int32_t)((j.M + v->bm - 1) / v->bm);
   p.tiles_n = (int32_t)((j.N + v->bn - 1) / v->bn);
