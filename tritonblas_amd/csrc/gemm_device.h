@@ -329,11 +329,11 @@ struct Frag {
       v4i lo = *(const v4i*)(rp + ((c0 ^ m) << 4));
       v4i hi = *(const v4i*)(rp + (((c0 + 1) ^ m) << 4));
       return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    } else if constexpr (T::DT == DT_FP4) {
-      int c = g * T::KSUB + ks;  // lane group g owns KSUB consecutive 32-blocks: their scale bytes are adjacent
-      return *(const v4i*)(rp + ((c ^ m) << 4));
     } else {
-      int c = ks * 4 + g;
+      // lane group g owns KSUB consecutive chunks.  fp4: their scale bytes are adjacent; all types:
+      // the four groups of one read then sit KSUB chunks apart, which spreads a wave's 64 addresses
+      // over the LDS banks (measured conflict-free, unlike groups reading four adjacent chunks).
+      int c = g * T::KSUB + ks;
       return *(const v4i*)(rp + ((c ^ m) << 4));
     }
   }
