@@ -8,6 +8,7 @@
 // Bit-level definition of the quantiser (must stay integer-exact):
 //   amax -> (bits + 0x200000) & 0xFF800000 -> e = exponent - 2, clamped to [-127, 127]
 //   scale byte = (e + 127) & 0xFF ; q = x * 2^-e ; code = round-half-up-in-magnitude(q), saturated to 6.0
+// The last step runs on v_cvt_scalef32_pk_fp4_f32 (two values per instruction); see the tie handling below.
 // This file is compiled with -ffp-contract=off: the rotation is fp32 adds/subs and one multiply.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -22,21 +23,6 @@ __device__ __forceinline__ float dpp_xor1(float v) {
 }
 __device__ __forceinline__ float dpp_xor2(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-}
-
-__device__ __forceinline__ uint32_t f32_to_e2m1(float q) {
-  uint32_t b = __builtin_bit_cast(uint32_t, q);
-  uint32_t s = b & 0x80000000u;
-  uint32_t e = (b >> 23) & 0xFFu;
-  uint32_t m = b & 0x7FFFFFu;
-  if (e < 127u) {
-    uint32_t adj = 126u - e;
-    m = (adj >= 32u) ? 0u : ((0x400000u | (m >> 1)) >> adj);
-  }
-  e = (e > 126u ? e : 126u) - 126u;
-  uint32_t t = (((e << 2) | (m >> 21)) + 1u) >> 1;
-  t = t < 7u ? t : 7u;
-  return (s >> 28) | t;
 }
 
 template <int XT>
@@ -126,9 +112,19 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
     // 2^-e as fp32 bits: normal for -e >= -126, the sub-normal 2^-127 for e = 127
     uint32_t qb = (e == 127) ? 0x00400000u : ((uint32_t)(127 - e) << 23);
     const float qs = __builtin_bit_cast(float, qb);
+    // e2m1 conversion on the hardware converter.  It rounds to nearest-even; the quantiser's rule is
+    // round-half-up in magnitude.  Setting the lowest fp32 mantissa bit moves every exact tie just
+    // above the tie point and changes no other rounding decision (tie points have zero low bits).
     uint32_t packed = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) packed |= f32_to_e2m1(x[i] * qs) << (4 * i);
+    for (int i = 0; i < 8; i += 2) {
+      const float q0 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[i] * qs) | 1u);
+      const float q1 = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x[i + 1] * qs) | 1u);
+      if (i == 0) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, q0, q1, 1.0f, 0);
+      if (i == 2) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, q0, q1, 1.0f, 1);
+      if (i == 4) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, q0, q1, 1.0f, 2);
+      if (i == 6) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, q0, q1, 1.0f, 3);
+    }
     if (ok[u]) {
       *(uint32_t*)(p.codes + row[u] * p.codes_stride + col[u] * 4) = packed;
       if (sub == 0) p.scales[row[u] * p.scales_stride + (col[u] >> 2)] = (uint8_t)((e + 127) & 0xFF);
