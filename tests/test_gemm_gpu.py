@@ -199,9 +199,14 @@ def test_streamk_explicit_grid(m, n, k, grid, dtype):
         _check(c.cpu(), want, dtype, TOL_16)
 
 
-def test_streamk_decode_shape_small():
-    """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly."""
+@pytest.mark.parametrize("kernel", ["streaming", "streamk"])
+def test_decode_shape_small(kernel, monkeypatch):
+    """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly:
+    through the streaming skinny-M kernel the library picks, and through the tile kernel's Stream-K
+    fixup (TB_NO_SKINNY switches the streaming kernel off)."""
     import tritonblas_amd as tb
+    if kernel == "streamk":
+        monkeypatch.setenv("TB_NO_SKINNY", "1")
     m, n, k = 32, 1024, 7168
     aq, bq, sa, sb = _a8w8_case(m, n, k, seed=21)
     a, b = aq.cuda(), bq.T.contiguous().cuda().T
@@ -212,6 +217,25 @@ def test_streamk_decode_shape_small():
         tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, cfg, enable_streamk=True)
     _check(c.cpu(), OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q)
     assert cfg.status() == 0
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+def test_skinny_rows(m, dtype):
+    """Every row-block count of the streaming kernel, ragged N, bias, all three element types."""
+    import tritonblas_amd as tb
+    n, k = 1040, 2304
+    _say(f"skinny {m}x{n}x{k} {dtype}")
+    if dtype == torch.float8_e4m3fn:
+        aq, bq, sa, sb = _a8w8_case(m, n, k, seed=31)
+        c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+        tb.matmul_a8w8(aq.cuda(), bq.T.contiguous().cuda().T, sa.cuda(), sb.cuda(), c)
+        _check(c.cpu(), OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q)
+    else:
+        a_cpu, b_cpu, bias = _rand((m, k), dtype, 32, 0.5), _rand((k, n), dtype, 33, 0.5), _rand((n,), dtype, 34)
+        b = b_cpu.T.contiguous().cuda().T
+        c = tb.addmm(bias.cuda(), a_cpu.cuda(), b)
+        _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32, bias=bias), dtype, TOL_16)
 
 
 # ---- MXFP4 --------------------------------------------------------------------------------------

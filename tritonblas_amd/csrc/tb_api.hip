@@ -10,6 +10,7 @@
 #include "../../include/tritonblas_amd.h"
 #include "gemm_variants.h"
 #include "quant.h"
+#include "skinny.h"
 #include "selector.h"
 
 using namespace tb;
@@ -132,6 +133,7 @@ struct Plan {
   const Variant* v = nullptr;
   GemmParams p;
   int grid = 0;
+  bool skinny = false;   // decode shapes: streaming kernel without tiles or workspace
   size_t ws_need = 0, ws_flags_off = 0, ws_p_off = 0, ws_counters_off = 0;
 };
 
@@ -246,6 +248,13 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
 
   const void* kern = (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) ? v->kernel_sk : v->kernel;
+  {
+    // a handful of rows against a K-major weight: the streaming kernel reads B once at HBM rate
+    const char* e = getenv("TB_NO_SKINNY");
+    plan->skinny = j.num_groups == 0 && skinny_supported(j.dt, j.M) && alay == LAY_K && blay == LAY_K &&
+                   KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !(e && atoi(e));
+    if (plan->skinny) { plan->v = v; plan->grid = 1; plan->ws_need = 0; return TB_OK; }
+  }
   const int occ = need_device ? kernel_occupancy(v, kern) : std::max(1, std::min(v->minb, hw.lds_bytes / v->lds_bytes));
   const int resident = hw.n_cu * occ;
   int grid;
@@ -289,6 +298,10 @@ int launch(const Job& j, hipStream_t stream) {
   st = make_plan(j, hw, true, &plan);
   if (st != TB_OK) return st;
   GemmParams& p = plan.p;
+  if (plan.skinny) {
+    if (launch_skinny(p, j.dt, stream) != hipSuccess) { (void)hipGetLastError(); return TB_ERR_LAUNCH; }
+    return TB_OK;
+  }
   if (plan.ws_need) {
     if (!j.workspace || j.workspace_bytes < plan.ws_need || ((uintptr_t)j.workspace & 255)) return TB_ERR_WORKSPACE;
     uint8_t* ws = (uint8_t*)j.workspace;

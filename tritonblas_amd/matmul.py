@@ -76,15 +76,15 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
         elif selector is not None and selector.streamk:
             d.grid = selector.sk_grid
     if schedule != _lib.TB_SCHED_PERSISTENT:
+        # 0 bytes: the library runs this problem with a kernel that needs no workspace (or refuses the
+        # descriptor, which the launch below reports)
         need = lib.tb_workspace_bytes(d)
-        if need == 0:
-            # the descriptor was refused; run the launch to surface the status
-            _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
-        if config is None:
-            config = MatmulConfig(device=dev, workspace=None, selector=selector)
-        ws = config.ensure(need)
-        d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
-        d.epoch = config.next_epoch()
+        if need > 0:
+            if config is None:
+                config = MatmulConfig(device=dev, workspace=None, selector=selector)
+            ws = config.ensure(need)
+            d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
+            d.epoch = config.next_epoch()
     with torch.cuda.device(dev):
         _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
     return c
