@@ -119,6 +119,13 @@ int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, in
     bool shorter_exists = false;
     for (int q = 0; q < ntiles; ++q) shorter_exists |= tiles[q].fast && tiles[q].bm < v.bm && tiles[q].bm >= pr.m;
     if (shorter_exists && pr.num_groups == 0) continue;
+    if (pr.num_groups > 0) {
+      // grouped: the row counts live on the device; size the tile for the average group so that the
+      // ragged last row block of each group wastes little
+      const int64_t avg = std::max<int64_t>(1, pr.m / pr.num_groups);
+      const int want = avg >= 192 ? 256 : (avg >= 96 ? 128 : 64);
+      if (v.bm != want || v.bn != want) continue;
+    }
     double c, m;
     double t = score(pr, hw, v, pr.streamk != 0, &c, &m);
     // prefer the larger tile on ties (less L2 traffic than the model resolves)

@@ -123,7 +123,12 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(const GemmParams p) 
 
 template <int DT, int MT>
 static hipError_t launch_mt(const GemmParams& p, hipStream_t stream) {
-  constexpr int NT = 2, WAVES = 8, DEPTH = 4;
+#ifndef SK_NT
+#define SK_NT 2
+#define SK_WAVES 8
+#define SK_DEPTH 4
+#endif
+  constexpr int NT = SK_NT, WAVES = SK_WAVES, DEPTH = SK_DEPTH;
   const int grid = (p.N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((skinny_kernel<DT, MT, NT, WAVES, DEPTH>), dim3(grid), dim3(WAVES * 64), 0, stream, p);
   return hipGetLastError();
