@@ -379,7 +379,9 @@ __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70);
 // ------------------------------------------------------------------------------------------------
 // K loop: accumulates k iterations [it0, it1) of one output tile
 // ------------------------------------------------------------------------------------------------
-template <class T>
+// WHOLE: the caller only ever passes complete tiles (it0 = 0, it1 = k_iters); lets the fp4 kernels
+// unroll the K loop over one scale group.
+template <class T, bool WHOLE>
 __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc, int it0, int it1,
                                          v4f (&acc)[T::TM][T::TN], uint8_t* lds, const LaneInfo& li) {
   using OA = Operand<T, T::BM, T::ALAY>;
@@ -420,7 +422,20 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
 
   // One K step of MFMAs from an LDS stage.  The A-side fragment of row block i+1 is requested before
   // the MFMAs of row block i are issued, so an LDS read is always in flight under the matrix pipe.
-  auto compute = [&](const uint8_t* sA, const uint8_t* sB) {
+  // fp4 kernels with LDS-staged scales keep the scale bytes of the SCG K steps of a group in ga/gb
+  // (8 bytes per lane and row block: step s, slice ks at byte s*KSUB+ks).  With a compile-time step
+  // position SC >= 0 the byte is picked by register index and op_sel; SC = -1 uses sca/scb.
+  constexpr bool MXG = (T::DT == DT_FP4) && T::DMA;
+  uint32_t ga[T::TM][2], gb[T::TN][2];
+#pragma unroll
+  for (int i = 0; i < T::TM; ++i) ga[i][0] = ga[i][1] = 0;
+#pragma unroll
+  for (int j = 0; j < T::TN; ++j) gb[j][0] = gb[j][1] = 0;
+
+  // One K step of MFMAs from an LDS stage.  The A-side fragment of row block i+1 is requested before
+  // the MFMAs of row block i are issued, so an LDS read is always in flight under the matrix pipe.
+  auto compute = [&](auto SC, const uint8_t* sA, const uint8_t* sB) {
+    constexpr int SCV = decltype(SC)::value;
 #pragma unroll
     for (int ks = 0; ks < T::KSUB; ++ks) {
       frag_t bf[T::TN];
@@ -435,10 +450,15 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         for (int j = 0; j < T::TN; ++j) {
           // output rows follow the first MFMA operand: feed B there so that one lane owns four
           // consecutive n of one m (contiguous in a row-major C).
-          if (ks == 0) acc[i][j] = mma<T, 0>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
-          if (ks == 1) acc[i][j] = mma<T, 1>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
-          if (ks == 2) acc[i][j] = mma<T, 2>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
-          if (ks == 3) acc[i][j] = mma<T, 3>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
+#define TB_MMA(KS)                                                                                             \
+  if (ks == KS) {                                                                                              \
+    constexpr bool ST = MXG && SCV >= 0;                                                                       \
+    constexpr int BYTE = ST ? (SCV * T::KSUB + KS) : KS;                                                       \
+    acc[i][j] = mma<T, (BYTE & 3)>(bf[j], af[i & 1], acc[i][j], ST ? gb[j][(BYTE >> 2) & 1] : scb[j],           \
+                                   ST ? ga[i][(BYTE >> 2) & 1] : sca[i]);                                       \
+  }
+          TB_MMA(0) TB_MMA(1) TB_MMA(2) TB_MMA(3)
+#undef TB_MMA
         }
       }
       // pin the issue order for the machine scheduler: B fragments and the first A fragment, then
@@ -457,11 +477,9 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
   if constexpr (T::DMA) {
     constexpr int S = T::STAGES;
     // Stage (it - it0) % S holds K step `it`; copies run S-1 steps ahead of the MFMAs.  One "group" is
-    // what a wave issues per K step: its share of both operand copies, then (fp4) its scale loads.
-    constexpr int NI = OA::NCH + OB::NCH;
-    constexpr int NSC = (T::DT == DT_FP4) ? (T::TM + T::TN) : 0;
-    constexpr int NG = NI + NSC;
-    static_assert((S - 2) * NG + NSC <= 63, "vmcnt range");
+    // what a wave issues per K step: its share of both operand copies.
+    constexpr int NG = OA::NCH + OB::NCH;
+    static_assert((S - 2) * NG <= 63, "vmcnt range");
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) {
       if (it0 + s < it1) {
@@ -469,16 +487,18 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
     }
-    // ---- MX scales through LDS (fp4): one group = the scale bytes of SCG K steps for every tile row ----
-    constexpr bool MXL = (T::DT == DT_FP4);
-    constexpr bool mx_lds = MXL;   // the fast fp4 kernels are only launched when the scale rows qualify
+    // ---- MX scales through LDS (fp4).  One scale group = 32 scale bytes of every tile row = the
+    // scales of SCG consecutive K steps.  A group is copied raw ([step][lane group][KSUB bytes] per
+    // row), transposed in place to [lane group][step][KSUB bytes] (8 contiguous bytes per lane group)
+    // and then read with one 8-byte LDS load per lane and row block.
     uint8_t* sc_lds = lds + T::LDS_BYTES;
     constexpr int NQ = (T::BM + T::BN) * (T::SC_GB / 16);          // 16-byte scale chunks per group
-    constexpr int NSCH = MXL ? (NQ + T::THREADS - 1) / T::THREADS : 1;
+    constexpr int NSCH = MXG ? (NQ + T::THREADS - 1) / T::THREADS : 1;
+    constexpr int NTR = MXG ? ((T::BM + T::BN) * 4 + T::THREADS - 1) / T::THREADS : 1;   // (row, lane group) items
     const uint8_t* scp[NSCH];
-    uint32_t ga[T::TM][2], gb[T::TN][2];
-    int reg_group = -1, lds_group = -1, read_it = -1;
-    if constexpr (MXL) {
+    int reg_group = -1, lds_group = -1, read_it = -1, dma_it = -1;
+    bool lds_ready = false;
+    if constexpr (MXG) {
 #pragma unroll
       for (int i = 0; i < NSCH; ++i) {
         const int q = i * T::THREADS + li.tid;
@@ -488,7 +508,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
     }
     auto sc_dma = [&](int grp) {
-      if constexpr (MXL) {
+      if constexpr (MXG) {
         const int wave_slot = __builtin_amdgcn_readfirstlane(li.tid & ~63);
         const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)sc_lds);
 #pragma unroll
@@ -500,34 +520,64 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         }
       }
     };
-    auto sc_read = [&]() {
-      if constexpr (MXL) {
-        auto rd = [&](int row, uint32_t(&out)[2]) {
-          const uint8_t* b = sc_lds + row * T::SC_GB + li.g * T::KSUB;
-          out[0] = out[1] = 0;
+    // in place: the four lanes that own one row are neighbours in a wave, and a wave's reads of an
+    // item all complete before its writes of that item are issued (the writes consume the reads)
+    auto sc_transpose = [&]() {
+      if constexpr (MXG) {
+        uint32_t w0[NTR], w1[NTR];
+#pragma unroll
+        for (int i = 0; i < NTR; ++i) {
+          const int idx = i * T::THREADS + li.tid;
+          w0[i] = w1[i] = 0;
+          if (((T::BM + T::BN) * 4) % T::THREADS != 0 && idx >= (T::BM + T::BN) * 4) continue;
+          const uint8_t* b = sc_lds + (idx >> 2) * T::SC_GB + (idx & 3) * T::KSUB;
 #pragma unroll
           for (int s = 0; s < T::SCG; ++s) {
             uint32_t v = (T::KSUB == 2) ? (uint32_t)(*(const uint16_t*)(b + s * T::CPR)) : (uint32_t)(*(b + s * T::CPR));
-            out[(s * T::KSUB) >> 2] |= v << (8 * ((s * T::KSUB) & 3));
+            if ((s * T::KSUB) >> 2) w1[i] |= v << (8 * ((s * T::KSUB) & 3));
+            else w0[i] |= v << (8 * ((s * T::KSUB) & 3));
           }
-        };
+        }
 #pragma unroll
-        for (int i = 0; i < T::TM; ++i) rd(li.wm0 + i * 16 + li.r, ga[i]);
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) rd(T::BM + li.wn0 + j * 16 + li.r, gb[j]);
+        for (int i = 0; i < NTR; ++i) {
+          const int idx = i * T::THREADS + li.tid;
+          if (((T::BM + T::BN) * 4) % T::THREADS != 0 && idx >= (T::BM + T::BN) * 4) continue;
+          *(uint2*)(sc_lds + (idx >> 2) * T::SC_GB + (idx & 3) * 8) = uint2{w0[i], w1[i]};
+        }
       }
     };
-    static_assert(!MXL || T::KSUB <= 2, "LDS-staged scales hold 8 bytes per lane and row block");
+    auto sc_read = [&]() {
+      if constexpr (MXG) {
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) {
+          uint2 v = *(const uint2*)(sc_lds + (li.wm0 + i * 16 + li.r) * T::SC_GB + li.g * 8);
+          ga[i][0] = v.x; ga[i][1] = v.y;
+        }
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+          uint2 v = *(const uint2*)(sc_lds + (T::BM + li.wn0 + j * 16 + li.r) * T::SC_GB + li.g * 8);
+          gb[j][0] = v.x; gb[j][1] = v.y;
+        }
+      }
+    };
+    static_assert(!MXG || T::KSUB <= 2, "LDS-staged scales hold 8 bytes per lane and row block");
 
-    if (mx_lds) { sc_dma(it0 / T::SCG); lds_group = it0 / T::SCG; }
+    if constexpr (MXG) { sc_dma(it0 / T::SCG); lds_group = it0 / T::SCG; }
     else load_scales(it0, sca, scb);
     wait_vm0();
     __syncthreads();
+    if constexpr (MXG) {
+      sc_transpose();
+      lds_ready = true;
+      __syncthreads();
+    }
     int stage = 0;
-    for (int it = it0; it < it1; ++it) {
+    // one K step; SC is the step's compile-time position in its scale group, or -1 (found at run time)
+    auto kstep = [&](int it, auto SC) {
+      constexpr int SCV = decltype(SC)::value;
       const int nxt = it + S - 1;
       int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
-      if (mx_lds) {
+      if constexpr (MXG) {
         const int grp = it / T::SCG;
         if (grp != reg_group) {
           if (lds_group != grp) {  // only right after a segment start: nobody could prefetch this group
@@ -535,28 +585,41 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
             wait_vm0();
             __syncthreads();
             lds_group = grp;
+            lds_ready = false;
+          }
+          if (!lds_ready) {
+            sc_transpose();
+            lds_ready = true;
+            __syncthreads();
           }
           sc_read();
           reg_group = grp;
           read_it = it;
-        } else if (it > read_it && lds_group == grp && (grp + 1) * T::SCG < it1) {
+        } else if (lds_group == grp && it > read_it && (grp + 1) * T::SCG < it1) {
           sc_dma(grp + 1);       // every wave has consumed group grp (a barrier has passed since)
           lds_group = grp + 1;
+          lds_ready = false;
+          dma_it = it;
+        } else if (lds_group == grp + 1 && !lds_ready && it > dma_it) {
+          sc_transpose();        // the copy landed with the wait that closed step dma_it
+          lds_ready = true;
         }
-        const int sidx = (it % T::SCG) * T::KSUB;
-        const int sh = 8 * (sidx & 3);
+        if constexpr (SCV < 0) {
+          const int sidx = (it % T::SCG) * T::KSUB;
+          const int sh = 8 * (sidx & 3);
 #pragma unroll
-        for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
+          for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
 #pragma unroll
-        for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
+          for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
+        }
       }
       if (nxt < it1 && !(p.debug & 1)) {
         OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
         OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
-      if (!mx_lds && it + 1 < it1) load_scales(it + 1, nsca, nscb);
-      if (!(p.debug & 2)) compute(lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
-      if (!mx_lds && it + 1 < it1) {
+      if (!MXG && it + 1 < it1) load_scales(it + 1, nsca, nscb);
+      if (!(p.debug & 2)) compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      if (!MXG && it + 1 < it1) {
 #pragma unroll
         for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
 #pragma unroll
@@ -564,7 +627,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
       // K step it+1 must have landed before the barrier; the S-2 younger groups may stay in flight.
       // (vmcnt counts in issue order; near the end of the tile fewer groups exist, so drain fully.)
-      if (S > 2 && nxt < it1 && !MXL) {
+      if (S > 2 && nxt < it1 && !MXG) {
         constexpr int ALLOWED = (S - 2) * NG;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
       } else {
@@ -572,6 +635,23 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
       __syncthreads();
       stage = (stage + 1 == S) ? 0 : stage + 1;
+    };
+    if constexpr (MXG && WHOLE) {
+      // whole tiles of the fast fp4 kernels: k_iters is a multiple of the scale group (K % 1024 == 0)
+      for (int it = it0; it < it1; it += T::SCG) {
+        kstep(it, std::integral_constant<int, 0>{});
+        kstep(it + 1, std::integral_constant<int, 1>{});
+        kstep(it + 2, std::integral_constant<int, 2>{});
+        kstep(it + 3, std::integral_constant<int, 3>{});
+        if constexpr (T::SCG == 8) {
+          kstep(it + 4, std::integral_constant<int, 4>{});
+          kstep(it + 5, std::integral_constant<int, 5>{});
+          kstep(it + 6, std::integral_constant<int, 6>{});
+          kstep(it + 7, std::integral_constant<int, 7>{});
+        }
+      }
+    } else {
+      for (int it = it0; it < it1; ++it) kstep(it, std::integral_constant<int, -1>{});
     }
   } else {
     v4i ra[OA::NREG], rb[OB::NREG];
@@ -591,7 +671,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::gload(rb, sb, it + 1, p.KU, li.tid);
         load_scales(it + 1, nsca, nscb);
       }
-      if (!(p.debug & 2)) compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
+      if (!(p.debug & 2)) compute(std::integral_constant<int, -1>{}, sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
       if (has_next) {
         OA::sstore(sA0 + (cur ^ 1) * T::STAGE_BYTES, ra, li.tid);
         OB::sstore(sB0 + (cur ^ 1) * T::STAGE_BYTES, rb, li.tid);
@@ -967,7 +1047,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   bool failed = false;
   while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
     __syncthreads();  // the previous item's store staging may still be read by slower waves
-    mainloop<T>(p, w.tc, w.it0, w.it1, acc, lds, li);
+    mainloop<T, !SK>(p, w.tc, w.it0, w.it1, acc, lds, li);
     if constexpr (SK) {
     if (w.kind == WK_SK_PUBLISH) {
       // not the tile's first segment: publish the partial, tagged with this launch's epoch
