@@ -49,7 +49,7 @@ def e8m0_to_f32(scale_e8m0: torch.Tensor) -> torch.Tensor:
     return bits.view(torch.float32)
 
 
-def _quant(x: torch.Tensor, hadamard: bool):
+def _quant(x: torch.Tensor, hadamard: bool, out=None):
     assert x.ndim == 2, "Input must be 2D tensor"
     M, N = x.shape
     assert N % 32 == 0, f"N ({N}) must be divisible by 32"
@@ -57,8 +57,14 @@ def _quant(x: torch.Tensor, hadamard: bool):
         raise RuntimeError("tritonblas_amd: the MXFP4 quantiser runs on the GPU only")
     if x.stride(1) != 1:
         x = x.contiguous()
-    codes = torch.empty((M, N // 2), dtype=torch.uint8, device=x.device)
-    scales = torch.empty((M, N // 32), dtype=torch.uint8, device=x.device)
+    if out is None:
+        codes = torch.empty((M, N // 2), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((M, N // 32), dtype=torch.uint8, device=x.device)
+    else:
+        codes, scales = out
+        for t, cols in ((codes, N // 2), (scales, N // 32)):
+            assert t.dtype == torch.uint8 and t.device == x.device and tuple(t.shape) == (M, cols) and t.stride(1) == 1, \
+                "out must be (codes (M, N/2), scales (M, N/32)) uint8 tensors on x's device with unit column stride"
     d = _lib.tb_quant_desc()
     d.struct_bytes = C.sizeof(_lib.tb_quant_desc)
     d.x_type = _lib.tb_dtype(x.dtype)
@@ -72,15 +78,15 @@ def _quant(x: torch.Tensor, hadamard: bool):
     return codes, scales
 
 
-def dynamic_mxfp4_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+def dynamic_mxfp4_quant(x: torch.Tensor, *, out=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """(M, N) fp32/fp16/bf16 -> (codes (M, N/2) uint8, E8M0 scales (M, N/32) uint8).
-    Reference utils.py:743-789."""
-    return _quant(x, hadamard=False)
+    Reference utils.py:743-789.  `out=(codes, scales)` writes into caller-owned tensors (no allocation)."""
+    return _quant(x, hadamard=False, out=out)
 
 
-def hadamard_mxfp4_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+def hadamard_mxfp4_quant(x: torch.Tensor, *, out=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Same, after rotating every block of 32 values along N by H32/sqrt(32) in the same kernel."""
-    return _quant(x, hadamard=True)
+    return _quant(x, hadamard=True, out=out)
 
 
 def hadamard32(x: torch.Tensor) -> torch.Tensor:
