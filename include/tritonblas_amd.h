@@ -46,7 +46,7 @@ enum {
 
 /* ---- schedules ------------------------------------------------------------------------------ */
 enum {
-  TB_SCHED_PERSISTENT = 0,    /* data parallel, one tile per workgroup   (matmul.py:160-198)        */
+  TB_SCHED_PERSISTENT = 0,    /* data parallel, resident grid loops over tiles (matmul.py:160-198)  */
   TB_SCHED_WORK_STEALING = 1, /* atomic tile queues per XCD x slot       (matmul.py:112-159)        */
   TB_SCHED_STREAMK = 2        /* data parallel tiles + Stream-K tail     (matmul.py:202-366)        */
 };
@@ -115,7 +115,7 @@ typedef struct tb_gemm_desc {
   int32_t block_m, block_n, block_k;  /* tile variant, from tb_select; 0 = let the library select    */
   int32_t group_m, num_xcds;
   int32_t schedule;           /* TB_SCHED_*                                                         */
-  int32_t grid;               /* Stream-K / work-stealing grid; 0 = default                         */
+  int32_t grid;               /* workgroups to launch; 0 = default (what is co-resident)            */
   int32_t counters_per_xcd;
   void* workspace;            /* tb_workspace_bytes() bytes, zero-initialised once by the caller     */
   size_t workspace_bytes;
@@ -186,6 +186,15 @@ typedef struct tb_quant_desc {
 } tb_quant_desc;
 
 int tb_hadamard_mxfp4_quant(const tb_quant_desc* desc, void* stream);
+
+/* ---- tile order ------------------------------------------------------------------------------
+ * Host-side evaluation of the kernels' tile id -> (row block, column block) map, for tests and tools.
+ * With panel_n = 0 it is the reference's GROUP_M swizzle (kernels/stages/schedule.py:124-145); with
+ * panel_n > 0 the tile list is cut into column panels of panel_n tiles that are each swept top to
+ * bottom with that swizzle (no counterpart in the reference: a cache-residency choice of this library).
+ * tb_default_panel gives the panel width tb_gemm uses for a launch grid. */
+int tb_tile_coords(int32_t tile, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t panel_n, int32_t* pm, int32_t* pn);
+int tb_default_panel(int32_t grid, int32_t chunk, int32_t group_m);
 
 /* ---- misc ----------------------------------------------------------------------------------- */
 const char* tb_status_string(int status);

@@ -146,3 +146,59 @@ def test_python_api_refuses_cpu_tensors():
         tb.matmul_lt(a, a, a.clone(), None, None)
     with pytest.raises(RuntimeError, match="differentiation"):
         tb.matmul(a.requires_grad_(), a, out=torch.zeros(16, 16, dtype=torch.float16))
+
+
+# ---- tile order of the kernels (host evaluation through the C ABI) -------------------------------
+import itertools
+
+
+def _load():
+    from tritonblas_amd import _lib
+    return _lib.load()
+
+
+def _coords(lib, t, tm, tn, gm, panel):
+    pm, pn = C.c_int32(-1), C.c_int32(-1)
+    assert lib.tb_tile_coords(t, tm, tn, gm, panel, C.byref(pm), C.byref(pn)) == 0
+    return pm.value, pn.value
+
+
+@pytest.mark.parametrize("tm,tn,gm", [(32, 112, 8), (4, 4, 8), (5, 7, 2), (1, 9, 8), (9, 1, 4), (13, 3, 8)])
+def test_tile_order_without_panels_is_the_reference_swizzle(tm, tn, gm):
+    from oracle import schedule as S
+    lib = _load()
+    for panel in (0, tn, tn + 5):
+        assert [_coords(lib, t, tm, tn, gm, panel) for t in range(tm * tn)] == [S.tile_coords(t, tm, tn, gm) for t in range(tm * tn)]
+
+
+@pytest.mark.parametrize("tm,tn,gm,panel", [(32, 112, 8, 16), (32, 112, 8, 32), (5, 7, 2, 3), (13, 30, 8, 4), (3, 9, 8, 1), (7, 10, 4, 9)])
+def test_tile_order_with_panels_is_a_bijection_panel_by_panel(tm, tn, gm, panel):
+    lib = _load()
+    got = [_coords(lib, t, tm, tn, gm, panel) for t in range(tm * tn)]
+    assert set(got) == set(itertools.product(range(tm), range(tn)))
+    # panels are visited left to right, each completely before the next; inside a panel the order is
+    # the reference swizzle of a (tm x width) problem
+    from oracle import schedule as S
+    pos = 0
+    for first in range(0, tn, panel):
+        width = min(panel, tn - first)
+        want = [(m, first + n) for (m, n) in (S.tile_coords(t, tm, width, gm) for t in range(tm * width))]
+        assert got[pos:pos + tm * width] == want
+        pos += tm * width
+
+
+def test_tile_coords_rejects_bad_arguments():
+    from tritonblas_amd._lib import TB_ERR_BAD_ARGUMENT, TB_ERR_NULL_POINTER
+    lib = _load()
+    pm, pn = C.c_int32(), C.c_int32()
+    assert lib.tb_tile_coords(12, 3, 4, 8, 0, C.byref(pm), C.byref(pn)) == TB_ERR_BAD_ARGUMENT
+    assert lib.tb_tile_coords(0, 3, 4, 0, 0, C.byref(pm), C.byref(pn)) == TB_ERR_BAD_ARGUMENT
+    assert lib.tb_tile_coords(0, 3, 4, 8, 0, None, C.byref(pn)) == TB_ERR_NULL_POINTER
+
+
+def test_default_panel_is_a_near_square_multiple_of_the_xcd_block():
+    lib = _load()
+    assert lib.tb_default_panel(256, 32, 8) == 16     # 8 XCD blocks of 8x4 tiles -> rounds of 16x16
+    assert lib.tb_default_panel(512, 64, 8) == 24
+    assert lib.tb_default_panel(1, 1, 1) == 1
+    assert lib.tb_default_panel(7, 1, 8) == 3

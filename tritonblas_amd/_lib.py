@@ -22,6 +22,7 @@ TB_SCHED_PERSISTENT, TB_SCHED_WORK_STEALING, TB_SCHED_STREAMK = 0, 1, 2
 EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
+    "tb_tile_coords", "tb_default_panel",
 ]
 
 
@@ -109,6 +110,8 @@ def load():
     lib.tb_gemm_fp4.argtypes = [C.POINTER(tb_gemm_fp4_desc), C.c_void_p]
     lib.tb_grouped_gemm_fp8.argtypes = [C.POINTER(tb_grouped_gemm_desc), C.c_void_p]
     lib.tb_hadamard_mxfp4_quant.argtypes = [C.POINTER(tb_quant_desc), C.c_void_p]
+    lib.tb_tile_coords.argtypes = [C.c_int32] * 5 + [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    lib.tb_default_panel.argtypes = [C.c_int32] * 3
     if lib.tb_abi_version() != 1:
         raise RuntimeError("libtritonblas_amd.so ABI version mismatch")
     _lib = lib

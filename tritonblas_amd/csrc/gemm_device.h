@@ -49,6 +49,7 @@ struct GemmParams {
   int32_t mx_lds;                // scale rows are 16-byte aligned and K/32 is a multiple of 32: stage scales in LDS
   int32_t tiles_m, tiles_n, total_tiles, k_iters;
   int32_t group_m, num_xcds, chunk;
+  int32_t panel_n;               // tile order: column panels of this many tiles, swept top to bottom (0: one panel)
   int32_t mode;
   int32_t debug;                 // tuning experiments: bit0 skip global->LDS copies, bit1 skip MFMA work
   // Stream-K
@@ -75,7 +76,7 @@ struct TileCtx {
 };
 
 template <int DT_, int BM_, int BN_, int BKB_, int WM_, int WN_, int ALAY_, int BLAY_, int MINB_ = 1,
-          bool FAST_ = true, int STAGES_ = 2, bool USE_DMA_ = true>
+          bool FAST_ = true, int STAGES_ = 2, bool USE_DMA_ = true, bool HALF_ = false>
 struct Tile {
   static constexpr int DT = DT_, BM = BM_, BN = BN_, BKB = BKB_, WM = WM_, WN = WN_;
   static constexpr int ALAY = ALAY_, BLAY = BLAY_, MINB = MINB_, STAGES = STAGES_;
@@ -97,13 +98,24 @@ struct Tile {
   static constexpr int TM = WTM / 16, TN = WTN / 16;
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  // HALF: one extra operand-sized LDS slot.  The copies then form a ring of 2*STAGES+1 slots
+  // (A0 B0 A1 B1 ...), the A operand runs one K step further ahead than B, and the copy queue never
+  // runs empty at the barrier that ends a K step.
+  static constexpr bool HALF = HALF_;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + (HALF ? A_BYTES : 0);
   // MX scales (fp4, LDS-direct kernels): 32 scale bytes per tile row are staged in LDS at a time,
   // i.e. the scales of SCG consecutive K steps (one 32-element block = one 16-byte chunk = one byte).
   static constexpr int SC_GB = 32;
   static constexpr int SCG = (DT == DT_FP4) ? SC_GB / CPR : 1;
   static constexpr int SC_BYTES = (DT == DT_FP4 && DMA) ? (BM + BN) * SC_GB : 0;
   static constexpr int LDS_TOTAL = LDS_BYTES + SC_BYTES;
+  static constexpr int LDS_LIMIT = 160 * 1024;
+  // the one word the schedules broadcast through LDS lives in the tile buffer's last 16 bytes when
+  // the buffer takes the whole LDS (it is only used between K loops)
+  static constexpr bool BCAST_IN_TILE = LDS_TOTAL + 16 > LDS_LIMIT;
+  static constexpr int LDS_ALLOC = BCAST_IN_TILE ? LDS_TOTAL : LDS_TOTAL + 16;
+  static_assert(LDS_TOTAL <= LDS_LIMIT, "tile buffers exceed the LDS of a CU");
+  static_assert(!HALF || (USE_DMA_ && FAST_ && ALAY_ == LAY_K && BLAY_ == LAY_K && BM_ == BN_), "half-stage ring: LDS-direct loader, equal operand tiles");
   static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // XOR-swizzle range of the chunk index
   static_assert(CPR % KS == 0, "K step must hold whole MFMA slices");
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be MFMA aligned");
@@ -132,14 +144,26 @@ __device__ __forceinline__ int chiplet_transform_chunked(int pid, int num_wg, in
   return chunk_idx * block + xcd * chunk + pos;
 }
 
-__device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int group_m, int& pm, int& pn) {
-  int in_group = group_m * tiles_n;
+// Tile id -> (row block, column block).  Column panels of panel_n tiles (the last may be narrower) are
+// visited one after the other; inside a panel, groups of group_m row blocks are swept left to right,
+// rows fastest.  Consecutive ids therefore share A row strips and B column strips, and a panel's B
+// strips are reused by every row group before the next panel starts.
+__host__ __device__ __forceinline__ void tile_coords(int tile, int tiles_m, int tiles_n, int group_m, int panel_n, int& pm, int& pn) {
+  int first_n = 0, width = tiles_n;
+  if (panel_n > 0 && panel_n < tiles_n) {
+    int per_panel = tiles_m * panel_n;
+    int pi = tile / per_panel;
+    first_n = pi * panel_n;
+    width = (tiles_n - first_n < panel_n) ? tiles_n - first_n : panel_n;
+    tile -= pi * per_panel;
+  }
+  int in_group = group_m * width;
   int gid = tile / in_group;
   int first = gid * group_m;
-  int gsz = min(tiles_m - first, group_m);
+  int gsz = (tiles_m - first < group_m) ? tiles_m - first : group_m;
   int rem = tile % in_group;
   pm = first + rem % gsz;
-  pn = rem / gsz;
+  pn = first_n + rem / gsz;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -328,13 +352,19 @@ struct Frag {
       int c0 = ks * 8 + 2 * g;
       v4i lo = *(const v4i*)(rp + ((c0 ^ m) << 4));
       v4i hi = *(const v4i*)(rp + (((c0 + 1) ^ m) << 4));
-      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      type f = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      // pin operand fragments to architectural VGPRs: kernels with one wave per SIMD keep their
+      // accumulators in the accumulation registers, and fragments placed there crowd them out
+      asm("" : "+v"(f));
+      return f;
     } else {
       // lane group g owns KSUB consecutive chunks.  fp4: their scale bytes are adjacent; all types:
       // the four groups of one read then sit KSUB chunks apart, which spreads a wave's 64 addresses
       // over the LDS banks (measured conflict-free, unlike groups reading four adjacent chunks).
       int c = g * T::KSUB + ks;
-      return *(const v4i*)(rp + ((c ^ m) << 4));
+      type f = *(const v4i*)(rp + ((c ^ m) << 4));
+      asm("" : "+v"(f));
+      return f;
     }
   }
 };
@@ -480,6 +510,8 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     // what a wave issues per K step: its share of both operand copies.
     constexpr int NG = OA::NCH + OB::NCH;
     static_assert((S - 2) * NG <= 63, "vmcnt range");
+    constexpr bool H = T::HALF;
+    constexpr int R = 2 * S + 1;          // ring slots (H)
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) {
       if (it0 + s < it1) {
@@ -487,6 +519,8 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
     }
+    const bool pro_half = H && it0 + S - 1 < it1;
+    if (pro_half) OA::dma(sa, it0 + S - 1, lds + (S - 1) * T::STAGE_BYTES, li.tid);
     // ---- MX scales through LDS (fp4).  One scale group = 32 scale bytes of every tile row = the
     // scales of SCG consecutive K steps.  A group is copied raw ([step][lane group][KSUB bytes] per
     // row), transposed in place to [lane group][step][KSUB bytes] (8 contiguous bytes per lane group)
@@ -564,19 +598,24 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
 
     if constexpr (MXG) { sc_dma(it0 / T::SCG); lds_group = it0 / T::SCG; }
     else load_scales(it0, sca, scb);
-    wait_vm0();
+    if (H && !MXG && T::DT != DT_FP4 && pro_half) __builtin_amdgcn_s_waitcnt(0x0F70 | (OA::NCH & 0xF) | ((OA::NCH >> 4) << 14));
+    else wait_vm0();
     __syncthreads();
     if constexpr (MXG) {
       sc_transpose();
       lds_ready = true;
       __syncthreads();
     }
-    int stage = 0;
+    int stage = 0;   // !H: stage of this K step; H: ring slot of its A operand (B follows)
     // one K step; SC is the step's compile-time position in its scale group, or -1 (found at run time)
     auto kstep = [&](int it, auto SC) {
       constexpr int SCV = decltype(SC)::value;
       const int nxt = it + S - 1;
       int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
+      int slot_b = stage + 1, slot_wb = stage - 2, slot_wa = stage - 1;   // H only
+      if (slot_b >= R) slot_b -= R;
+      if (slot_wb < 0) slot_wb += R;
+      if (slot_wa < 0) slot_wa += R;
       if constexpr (MXG) {
         const int grp = it / T::SCG;
         if (grp != reg_group) {
@@ -613,12 +652,21 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
           for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
         }
       }
-      if (nxt < it1 && !(p.debug & 1)) {
-        OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
-        OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
+      if constexpr (H) {
+        // the slots of step it-1 are free: B of step it+S-1, then A of step it+S
+        if (nxt < it1 && !(p.debug & 1)) OB::dma(sb, nxt, lds + slot_wb * T::A_BYTES, li.tid);
+        if (nxt + 1 < it1 && !(p.debug & 1)) OA::dma(sa, nxt + 1, lds + slot_wa * T::A_BYTES, li.tid);
+      } else {
+        if (nxt < it1 && !(p.debug & 1)) {
+          OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
+          OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
+        }
       }
       if (!MXG && it + 1 < it1) load_scales(it + 1, nsca, nscb);
-      if (!(p.debug & 2)) compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      if (!(p.debug & 2)) {
+        if constexpr (H) compute(SC, lds + stage * T::A_BYTES, lds + slot_b * T::A_BYTES);
+        else compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      }
       if (!MXG && it + 1 < it1) {
 #pragma unroll
         for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
@@ -627,14 +675,22 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
       // K step it+1 must have landed before the barrier; the S-2 younger groups may stay in flight.
       // (vmcnt counts in issue order; near the end of the tile fewer groups exist, so drain fully.)
-      if (S > 2 && nxt < it1 && !MXG) {
+      // With the half-stage ring the A copy of step it+S may stay in flight as well.  fp4 kernels
+      // without LDS-staged scales load scales through registers (also vmcnt): they drain fully.
+      constexpr bool COUNTED = !MXG && T::DT != DT_FP4;
+      if (COUNTED && H && nxt + 1 < it1) {
+        constexpr int ALLOWED = (S - 2) * NG + OA::NCH;
+        static_assert(ALLOWED <= 63, "vmcnt range");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
+      } else if (COUNTED && !H && S > 2 && nxt < it1) {
         constexpr int ALLOWED = (S - 2) * NG;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
       } else {
         wait_vm0();
       }
       __syncthreads();
-      stage = (stage + 1 == S) ? 0 : stage + 1;
+      if constexpr (H) { stage += 2; if (stage >= R) stage -= R; }
+      else stage = (stage + 1 == S) ? 0 : stage + 1;
     };
     if constexpr (MXG && WHOLE) {
       // whole tiles of the fast fp4 kernels: k_iters is a multiple of the scale group (K % 1024 == 0)
@@ -775,6 +831,7 @@ __device__ __forceinline__ void epilogue_lines(const GemmParams& p, const TileCt
   constexpr int MAXROWS = (T::LDS_BYTES / WAVES / RS) / 16 * 16;
   constexpr int PASS_TM = (MAXROWS / 16 >= T::TM) ? T::TM : MAXROWS / 16;   // row blocks per pass
   static_assert(PASS_TM >= 1, "LDS too small for the store staging");
+  static_assert(WAVES * PASS_TM * 16 * RS <= T::LDS_ALLOC - 16, "store staging must leave the broadcast word alone");
   constexpr int CPRW = ROWB / 16;              // 16-byte chunks per row
   constexpr int ROWS_PER_INST = 64 / CPRW;
   uint8_t* stage = lds + (li.tid >> 6) * (PASS_TM * 16 * RS);
@@ -910,7 +967,7 @@ struct Work {
 
 __device__ __forceinline__ void plain_tile(const GemmParams& p, int tile, int BM, int BN, TileCtx& tc) {
   int pm, pn;
-  tile_coords(tile, p.tiles_m, p.tiles_n, p.group_m, pm, pn);
+  tile_coords(tile, p.tiles_m, p.tiles_n, p.group_m, p.panel_n, pm, pn);
   tc.m0 = pm * BM; tc.n0 = pn * BN; tc.m_lim = p.M; tc.n_lim = p.N;
   tc.B = p.B; tc.sb = p.sb;
 }
@@ -1029,8 +1086,8 @@ struct Sched {
 // the accumulator-heavy fixup code cannot push the common path into register spills.
 template <class T, bool SK>
 __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmParams p) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_TOTAL];
-  __shared__ int s_bcast;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_ALLOC];
+  int& s_bcast = *(int*)(lds + T::LDS_ALLOC - 16);
   LaneInfo li;
   li.tid = threadIdx.x;
   li.lane = li.tid & 63;

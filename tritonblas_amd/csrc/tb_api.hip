@@ -91,18 +91,30 @@ std::vector<TileInfo> tile_infos(int dt) {
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
-  // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
+  // tuning hook: TB_WAVES=<wm><wn>[<stages>[<half>]] picks among variants that share a tile shape
   const char* wenv = getenv("TB_WAVES");
   const int want = wenv ? atoi(wenv) : 0;
   if (want && fast)
     for (int i = 0; i < n; ++i)
       if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
-          (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want))
+          (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want ||
+           v[i].wm * 1000 + v[i].wn * 100 + v[i].stages * 10 + v[i].half == want))
         return &v[i];
   for (int i = 0; i < n; ++i)
     if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk)))
       return &v[i];
   return nullptr;
+}
+
+// Width (in tiles) of the column panels of the tile order.  One pass of the grid over the tile list
+// ("round") should cover a near-square block of C, so that the A and B strips a round needs are few and
+// shared by many workgroups, and the panel's B strips are reused by every row group before they leave
+// the memory-side cache.  A multiple of the width of one XCD's block (chunk / group_m columns).
+int default_panel_n(int grid, int chunk, int group_m) {
+  const int bw = std::max(1, chunk / std::max(1, group_m));
+  int side = 1;
+  while (side * side < grid) ++side;
+  return std::max(bw, (side + bw - 1) / bw * bw);
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -263,8 +275,10 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     p.mode = MODE_GROUPED;
     grid = (int)(((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n);
   } else if (j.schedule == TB_SCHED_PERSISTENT) {
+    // a resident grid that loops over the tiles (matmul.py:160-198: for tile_id in range(pid, total, NUM_SMS))
     p.mode = MODE_STATIC;
-    grid = p.total_tiles;
+    grid = (int)std::min<int64_t>(total, j.grid > 0 ? j.grid : resident);
+    { const char* e = getenv("TB_GRID"); if (e && atoi(e) > 0) grid = (int)std::min<int64_t>(total, atoi(e)); }
   } else if (j.schedule == TB_SCHED_WORK_STEALING) {
     p.mode = MODE_WS;
     grid = j.grid > 0 ? j.grid : resident;
@@ -285,6 +299,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   }
   if (grid <= 0) return TB_ERR_BAD_SHAPE;
   p.chunk = std::min(p.group_m * p.group_m, std::max(1, grid / p.num_xcds));
+  p.panel_n = default_panel_n(grid, p.chunk, p.group_m);
+  { const char* e = getenv("TB_PANEL"); if (e) p.panel_n = atoi(e); }
   plan->grid = grid;
   plan->v = v;
   return TB_OK;
@@ -340,6 +356,20 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
 extern "C" {
 
 int tb_abi_version(void) { return TB_ABI_VERSION; }
+
+int tb_tile_coords(int32_t tile, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t panel_n, int32_t* pm, int32_t* pn) {
+  if (!pm || !pn) return TB_ERR_NULL_POINTER;
+  if (tiles_m <= 0 || tiles_n <= 0 || group_m <= 0 || panel_n < 0 || tile < 0 || (int64_t)tile >= (int64_t)tiles_m * tiles_n) return TB_ERR_BAD_ARGUMENT;
+  int m, n;
+  tile_coords(tile, tiles_m, tiles_n, group_m, panel_n, m, n);
+  *pm = m; *pn = n;
+  return TB_OK;
+}
+
+int tb_default_panel(int32_t grid, int32_t chunk, int32_t group_m) {
+  if (grid <= 0 || chunk <= 0 || group_m <= 0) return TB_ERR_BAD_ARGUMENT;
+  return default_panel_n(grid, chunk, group_m);
+}
 
 const char* tb_status_string(int status) {
   switch (status) {
