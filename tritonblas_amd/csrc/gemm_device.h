@@ -76,7 +76,7 @@ struct TileCtx {
 };
 
 template <int DT_, int BM_, int BN_, int BKB_, int WM_, int WN_, int ALAY_, int BLAY_, int MINB_ = 1,
-          bool FAST_ = true, int STAGES_ = 2, bool USE_DMA_ = true, bool HALF_ = false>
+          bool FAST_ = true, int STAGES_ = 2, bool USE_DMA_ = true>
 struct Tile {
   static constexpr int DT = DT_, BM = BM_, BN = BN_, BKB = BKB_, WM = WM_, WN = WN_;
   static constexpr int ALAY = ALAY_, BLAY = BLAY_, MINB = MINB_, STAGES = STAGES_;
@@ -98,11 +98,7 @@ struct Tile {
   static constexpr int TM = WTM / 16, TN = WTN / 16;
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  // HALF: one extra operand-sized LDS slot.  The copies then form a ring of 2*STAGES+1 slots
-  // (A0 B0 A1 B1 ...), the A operand runs one K step further ahead than B, and the copy queue never
-  // runs empty at the barrier that ends a K step.
-  static constexpr bool HALF = HALF_;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + (HALF ? A_BYTES : 0);
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   // MX scales (fp4, LDS-direct kernels): 32 scale bytes per tile row are staged in LDS at a time,
   // i.e. the scales of SCG consecutive K steps (one 32-element block = one 16-byte chunk = one byte).
   static constexpr int SC_GB = 32;
@@ -115,7 +111,6 @@ struct Tile {
   static constexpr bool BCAST_IN_TILE = LDS_TOTAL + 16 > LDS_LIMIT;
   static constexpr int LDS_ALLOC = BCAST_IN_TILE ? LDS_TOTAL : LDS_TOTAL + 16;
   static_assert(LDS_TOTAL <= LDS_LIMIT, "tile buffers exceed the LDS of a CU");
-  static_assert(!HALF || (USE_DMA_ && FAST_ && ALAY_ == LAY_K && BLAY_ == LAY_K && BM_ == BN_), "half-stage ring: LDS-direct loader, equal operand tiles");
   static constexpr int SWM = (CPR >= 16) ? 16 : CPR;       // XOR-swizzle range of the chunk index
   static_assert(CPR % KS == 0, "K step must hold whole MFMA slices");
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be MFMA aligned");
@@ -352,19 +347,13 @@ struct Frag {
       int c0 = ks * 8 + 2 * g;
       v4i lo = *(const v4i*)(rp + ((c0 ^ m) << 4));
       v4i hi = *(const v4i*)(rp + (((c0 + 1) ^ m) << 4));
-      type f = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      // pin operand fragments to architectural VGPRs: kernels with one wave per SIMD keep their
-      // accumulators in the accumulation registers, and fragments placed there crowd them out
-      asm("" : "+v"(f));
-      return f;
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     } else {
       // lane group g owns KSUB consecutive chunks.  fp4: their scale bytes are adjacent; all types:
       // the four groups of one read then sit KSUB chunks apart, which spreads a wave's 64 addresses
       // over the LDS banks (measured conflict-free, unlike groups reading four adjacent chunks).
       int c = g * T::KSUB + ks;
-      type f = *(const v4i*)(rp + ((c ^ m) << 4));
-      asm("" : "+v"(f));
-      return f;
+      return *(const v4i*)(rp + ((c ^ m) << 4));
     }
   }
 };
@@ -504,14 +493,134 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     }
   };
 
-  if constexpr (T::DMA) {
+  if constexpr (T::DMA && !MXG) {
     constexpr int S = T::STAGES;
-    // Stage (it - it0) % S holds K step `it`; copies run S-1 steps ahead of the MFMAs.  One "group" is
-    // what a wave issues per K step: its share of both operand copies.
+    // Stage (it - it0) % S holds K step `it`.  One "group" is what a wave issues per K step: its share
+    // of both operand copies.  All S stages are filled up front; afterwards the copy of step it+S is
+    // issued in the middle of step `it`, right after the barrier that frees that step's stage.
+    constexpr int NG = OA::NCH + OB::NCH;
+    static_assert((S - 1) * NG <= 63, "vmcnt range");
+    int issued = 0;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      if (it0 + s < it1) {
+        OA::dma(sa, it0 + s, lds + s * T::STAGE_BYTES, li.tid);
+        OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
+        ++issued;
+      }
+    }
+    // step it0 must have landed; the younger stages may stay in flight (vmcnt counts in issue order)
+    if (issued == S) __builtin_amdgcn_s_waitcnt(0x0F70 | (((S - 1) * NG) & 0xF) | ((((S - 1) * NG) >> 4) << 14));
+    else wait_vm0();
+    __syncthreads();
+
+    // ---- software pipeline over (K step, MFMA slice) blocks ------------------------------------
+    // On entry to a block its B fragments and its first A fragment are already in registers: they
+    // were requested under the last row block of MFMAs of the block before.  Inside a block the A
+    // fragment of row block i+1 is requested before the MFMAs of row block i.  The barrier that ends
+    // a K step therefore sits in front of the last row block of its last slice, whose operands are
+    // in registers: after it the freed stage is refilled, the next step's fragments are requested,
+    // and the matrix pipe has that row block to chew on while they arrive.
+    frag_t bf[T::TN];
+    frag_t afn;
+    auto request_b = [&](const uint8_t* sB, int ks, int j) { bf[j] = Frag<T>::read(sB, li.wn0 + j * 16 + li.r, ks, li.g, swm); };
+    auto request_a = [&](const uint8_t* sA, int ks, int i) { return Frag<T>::read(sA, li.wm0 + i * 16 + li.r, ks, li.g, swm); };
+    constexpr int RPF = (T::DT == DT_FP8) ? 2 : 1;  // LDS reads per fragment
+
+    // one block: slice KSV of the K step in stage (sA, sB).  `boundary` runs before the last row block;
+    // afterwards the fragments of slice nks of stage (nA, nB) are requested.  After the last step of
+    // the range that request still runs (no branch in the pipeline): it reads whatever the next stage
+    // holds and nobody uses the result.
+    auto block = [&](auto KSC, const uint8_t* sA, auto&& boundary, const uint8_t* nA, const uint8_t* nB, int nks) {
+      constexpr int KSV = decltype(KSC)::value;
+      frag_t af[2];
+      af[0] = afn;
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) {
+        if (i + 1 < T::TM) af[(i + 1) & 1] = request_a(sA, KSV, i + 1);
+        if (i + 1 == T::TM) {
+          // pin the issue order so far for the machine scheduler (the barrier inside `boundary` ends
+          // a scheduling region): one fragment request, then one row block of MFMAs
+#pragma unroll
+          for (int q = 0; q + 1 < T::TM; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, T::TN, 0);
+          }
+          boundary();
+          afn = request_a(nA, nks, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+          // output rows follow the first MFMA operand: feed B there so that one lane owns four
+          // consecutive n of one m (contiguous in a row-major C).
+          acc[i][j] = mma<T, 0>(bf[j], af[i & 1], acc[i][j], 0u, 0u);
+          if (i + 1 == T::TM) request_b(nB, nks, j);
+        }
+      }
+      // last row block: the next A fragment, then MFMAs and B fragment requests alternate
+      __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+      }
+    };
+
+    // fragments of the first block
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) request_b(lds + T::A_BYTES, 0, j);
+    afn = request_a(lds, 0, 0);
+
+    int stage = 0;
+    auto kstep = [&](int it) {
+      int nstage = (stage + 1 == S) ? 0 : stage + 1;
+      const uint8_t* sA = lds + stage * T::STAGE_BYTES;
+      const uint8_t* sB = sA + T::A_BYTES;
+      const uint8_t* nA = lds + nstage * T::STAGE_BYTES;
+      const uint8_t* nB = nA + T::A_BYTES;
+      // end of the K step: step it+1 must have landed (the S-2 younger copies may stay in flight while
+      // they all exist; near the end of the range drain fully), every wave must be done reading this
+      // stage, then the stage takes the copy of step it+S
+      auto boundary = [&]() {
+        // (lgkmcnt(0): this wave's reads of the stage have returned before anyone may overwrite it)
+        if (S > 2 && it + S - 1 < it1) {
+          constexpr int ALLOWED = (S - 2) * NG;
+          __builtin_amdgcn_s_waitcnt(0x0070 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0070);
+        }
+        __syncthreads();
+        if (it + S < it1 && !(p.debug & 1)) {
+          OA::dma(sa, it + S, lds + stage * T::STAGE_BYTES, li.tid);
+          OB::dma(sb, it + S, lds + stage * T::STAGE_BYTES + T::A_BYTES, li.tid);
+        }
+      };
+      auto nothing = []() {};
+      if (p.debug & 2) {
+        boundary();
+      } else {
+        if constexpr (T::KSUB == 1) {
+          block(std::integral_constant<int, 0>{}, sA, boundary, nA, nB, 0);
+        } else if constexpr (T::KSUB == 2) {
+          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1);
+          block(std::integral_constant<int, 1>{}, sA, boundary, nA, nB, 0);
+        } else {
+          static_assert(T::KSUB == 4, "MFMA slices per K step");
+          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1);
+          block(std::integral_constant<int, 1>{}, sA, nothing, sA, sB, 2);
+          block(std::integral_constant<int, 2>{}, sA, nothing, sA, sB, 3);
+          block(std::integral_constant<int, 3>{}, sA, boundary, nA, nB, 0);
+        }
+      }
+      stage = nstage;
+    };
+    for (int it = it0; it < it1; ++it) kstep(it);
+  } else if constexpr (T::DMA) {
+    // fp4 with LDS-staged scales: copies run S-1 steps ahead, one barrier at the end of every K step
+    // (the scale registers leave no room for fragments that live across the barrier).
+    constexpr int S = T::STAGES;
     constexpr int NG = OA::NCH + OB::NCH;
     static_assert((S - 2) * NG <= 63, "vmcnt range");
-    constexpr bool H = T::HALF;
-    constexpr int R = 2 * S + 1;          // ring slots (H)
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) {
       if (it0 + s < it1) {
@@ -519,8 +628,6 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
     }
-    const bool pro_half = H && it0 + S - 1 < it1;
-    if (pro_half) OA::dma(sa, it0 + S - 1, lds + (S - 1) * T::STAGE_BYTES, li.tid);
     // ---- MX scales through LDS (fp4).  One scale group = 32 scale bytes of every tile row = the
     // scales of SCG consecutive K steps.  A group is copied raw ([step][lane group][KSUB bytes] per
     // row), transposed in place to [lane group][step][KSUB bytes] (8 contiguous bytes per lane group)
@@ -596,103 +703,63 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     };
     static_assert(!MXG || T::KSUB <= 2, "LDS-staged scales hold 8 bytes per lane and row block");
 
-    if constexpr (MXG) { sc_dma(it0 / T::SCG); lds_group = it0 / T::SCG; }
-    else load_scales(it0, sca, scb);
-    if (H && !MXG && T::DT != DT_FP4 && pro_half) __builtin_amdgcn_s_waitcnt(0x0F70 | (OA::NCH & 0xF) | ((OA::NCH >> 4) << 14));
-    else wait_vm0();
+    sc_dma(it0 / T::SCG);
+    lds_group = it0 / T::SCG;
+    wait_vm0();
     __syncthreads();
-    if constexpr (MXG) {
-      sc_transpose();
-      lds_ready = true;
-      __syncthreads();
-    }
-    int stage = 0;   // !H: stage of this K step; H: ring slot of its A operand (B follows)
+    sc_transpose();
+    lds_ready = true;
+    __syncthreads();
+    int stage = 0;
     // one K step; SC is the step's compile-time position in its scale group, or -1 (found at run time)
     auto kstep = [&](int it, auto SC) {
       constexpr int SCV = decltype(SC)::value;
       const int nxt = it + S - 1;
       int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
-      int slot_b = stage + 1, slot_wb = stage - 2, slot_wa = stage - 1;   // H only
-      if (slot_b >= R) slot_b -= R;
-      if (slot_wb < 0) slot_wb += R;
-      if (slot_wa < 0) slot_wa += R;
-      if constexpr (MXG) {
-        const int grp = it / T::SCG;
-        if (grp != reg_group) {
-          if (lds_group != grp) {  // only right after a segment start: nobody could prefetch this group
-            sc_dma(grp);
-            wait_vm0();
-            __syncthreads();
-            lds_group = grp;
-            lds_ready = false;
-          }
-          if (!lds_ready) {
-            sc_transpose();
-            lds_ready = true;
-            __syncthreads();
-          }
-          sc_read();
-          reg_group = grp;
-          read_it = it;
-        } else if (lds_group == grp && it > read_it && (grp + 1) * T::SCG < it1) {
-          sc_dma(grp + 1);       // every wave has consumed group grp (a barrier has passed since)
-          lds_group = grp + 1;
+      const int grp = it / T::SCG;
+      if (grp != reg_group) {
+        if (lds_group != grp) {  // only right after a segment start: nobody could prefetch this group
+          sc_dma(grp);
+          wait_vm0();
+          __syncthreads();
+          lds_group = grp;
           lds_ready = false;
-          dma_it = it;
-        } else if (lds_group == grp + 1 && !lds_ready && it > dma_it) {
-          sc_transpose();        // the copy landed with the wait that closed step dma_it
+        }
+        if (!lds_ready) {
+          sc_transpose();
           lds_ready = true;
+          __syncthreads();
         }
-        if constexpr (SCV < 0) {
-          const int sidx = (it % T::SCG) * T::KSUB;
-          const int sh = 8 * (sidx & 3);
+        sc_read();
+        reg_group = grp;
+        read_it = it;
+      } else if (lds_group == grp && it > read_it && (grp + 1) * T::SCG < it1) {
+        sc_dma(grp + 1);       // every wave has consumed group grp (a barrier has passed since)
+        lds_group = grp + 1;
+        lds_ready = false;
+        dma_it = it;
+      } else if (lds_group == grp + 1 && !lds_ready && it > dma_it) {
+        sc_transpose();        // the copy landed with the wait that closed step dma_it
+        lds_ready = true;
+      }
+      if constexpr (SCV < 0) {
+        const int sidx = (it % T::SCG) * T::KSUB;
+        const int sh = 8 * (sidx & 3);
 #pragma unroll
-          for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
+        for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
 #pragma unroll
-          for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
-        }
+        for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
       }
-      if constexpr (H) {
-        // the slots of step it-1 are free: B of step it+S-1, then A of step it+S
-        if (nxt < it1 && !(p.debug & 1)) OB::dma(sb, nxt, lds + slot_wb * T::A_BYTES, li.tid);
-        if (nxt + 1 < it1 && !(p.debug & 1)) OA::dma(sa, nxt + 1, lds + slot_wa * T::A_BYTES, li.tid);
-      } else {
-        if (nxt < it1 && !(p.debug & 1)) {
-          OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
-          OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
-        }
+      if (nxt < it1 && !(p.debug & 1)) {
+        OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
+        OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
       }
-      if (!MXG && it + 1 < it1) load_scales(it + 1, nsca, nscb);
-      if (!(p.debug & 2)) {
-        if constexpr (H) compute(SC, lds + stage * T::A_BYTES, lds + slot_b * T::A_BYTES);
-        else compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
-      }
-      if (!MXG && it + 1 < it1) {
-#pragma unroll
-        for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j];
-      }
-      // K step it+1 must have landed before the barrier; the S-2 younger groups may stay in flight.
-      // (vmcnt counts in issue order; near the end of the tile fewer groups exist, so drain fully.)
-      // With the half-stage ring the A copy of step it+S may stay in flight as well.  fp4 kernels
-      // without LDS-staged scales load scales through registers (also vmcnt): they drain fully.
-      constexpr bool COUNTED = !MXG && T::DT != DT_FP4;
-      if (COUNTED && H && nxt + 1 < it1) {
-        constexpr int ALLOWED = (S - 2) * NG + OA::NCH;
-        static_assert(ALLOWED <= 63, "vmcnt range");
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
-      } else if (COUNTED && !H && S > 2 && nxt < it1) {
-        constexpr int ALLOWED = (S - 2) * NG;
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (ALLOWED & 0xF) | ((ALLOWED >> 4) << 14));
-      } else {
-        wait_vm0();
-      }
+      if (!(p.debug & 2)) compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
+      wait_vm0();   // (the scale copy is the youngest load of a step: nothing may stay in flight)
       __syncthreads();
-      if constexpr (H) { stage += 2; if (stage >= R) stage -= R; }
-      else stage = (stage + 1 == S) ? 0 : stage + 1;
+      stage = (stage + 1 == S) ? 0 : stage + 1;
     };
-    if constexpr (MXG && WHOLE) {
+    if constexpr (WHOLE) {
       // whole tiles of the fast fp4 kernels: k_iters is a multiple of the scale group (K % 1024 == 0)
       for (int it = it0; it < it1; it += T::SCG) {
         kstep(it, std::integral_constant<int, 0>{});

@@ -10,7 +10,6 @@ struct Variant {
   int alay, blay;         // operand loaders (LAY_K / LAY_M)
   int wm, wn, threads, lds_bytes, minb;
   int fast, stages;       // fast: vector/LDS-direct loaders (alignment + K multiple required)
-  int half;               // extra operand-sized LDS slot (copy ring of 2*stages+1 slots)
   const void* kernel;     // __global__ void (*)(const GemmParams), whole-tile schedules
   const void* kernel_sk;  // same tile with the Stream-K tail
 };
@@ -18,7 +17,7 @@ struct Variant {
 template <class T>
 constexpr Variant make_variant() {
   return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_ALLOC, T::MINB,
-                 T::FAST ? 1 : 0, T::STAGES, T::HALF ? 1 : 0, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>};
+                 T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>};
 }
 
 // defined one per translation unit

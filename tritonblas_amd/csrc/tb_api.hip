@@ -91,14 +91,13 @@ std::vector<TileInfo> tile_infos(int dt) {
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
-  // tuning hook: TB_WAVES=<wm><wn>[<stages>[<half>]] picks among variants that share a tile shape
+  // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
   const char* wenv = getenv("TB_WAVES");
   const int want = wenv ? atoi(wenv) : 0;
   if (want && fast)
     for (int i = 0; i < n; ++i)
       if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
-          (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want ||
-           v[i].wm * 1000 + v[i].wn * 100 + v[i].stages * 10 + v[i].half == want))
+          (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want))
         return &v[i];
   for (int i = 0; i < n; ++i)
     if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk)))
