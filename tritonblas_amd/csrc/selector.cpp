@@ -52,17 +52,24 @@ int variant_occupancy(const TileInfo& v, const tb_hw& hw) {
   return std::max(1, std::min({by_lds, by_waves, v.minb}));
 }
 
-// Measured behaviour of the built kernels on MI355X that the model is anchored to:
-//   * MFMA-side efficiency of the K loop with operands already in LDS (fraction of the matrix pipe):
-//     256x256 tiles ~0.47, 128x128 ~0.64, 64x64 ~0.55, the skinny 32x128 tile ~0.30;
-//   * L2 -> LDS fill rate per CU: ~16 B/clk with one workgroup per CU, ~30 B/clk with two or more
-//     (the vector L1 keeps a bounded number of lines in flight, so the rate is latency-bound).
-static double mfma_side_efficiency(const TileInfo& v) {
+// Measured behaviour of the built kernels on MI355X that the model is anchored to (8192-class
+// problems for the saturated rates, 128..2048-row problems for the latency floor):
+//   * a CU that is kept busy by `occ` resident workgroups finishes one K step of one tile every
+//     ideal_step / eff: eff = fraction of the MFMA peak the kernel family sustains for that tile area;
+//   * a workgroup cannot turn a K step around faster than ~0.3 us (barrier + L2 round trip) plus the
+//     time its own copy takes at the ~100 GB/s one workgroup pulls (0.46 us for a 16 KB step, 0.65 us
+//     for 40 KB): small problems want enough tiles to put several workgroups on every CU, and
+//     long-K problems with few rows want the deep 32x128x256 tile;
+//   * per tile: epilogue + first-copy latency, ~12 us for 256x256, ~4 us for 128x128, ~3 us below.
+static double family_efficiency(int dt, const TileInfo& v) {
   const int area = v.bm * v.bn;
-  if (area >= 256 * 256) return 0.47;
-  if (area >= 128 * 128) return 0.64;
-  if (area >= 64 * 64) return 0.55;
-  return 0.30;
+  const int cls = (v.bm < 64 || v.bn < 64) ? 3 : (area >= 256 * 256 ? 0 : (area >= 128 * 128 ? 1 : 2));
+  static const double f8[4] = {0.61, 0.52, 0.29, 0.15};
+  static const double h16[4] = {0.59, 0.50, 0.22, 0.12};
+  static const double f4[4] = {0.45, 0.36, 0.22, 0.10};
+  if (dt == TB_FP8_E4M3) return f8[cls];
+  if (dt == TB_FP4_E2M1) return f4[cls];
+  return h16[cls];
 }
 
 static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk, double* comp_us,
@@ -74,30 +81,30 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   const int64_t tiles = tiles_m * tiles_n + (pr.num_groups > 0 ? (int64_t)pr.num_groups * tiles_n / 2 : 0);
   const int64_t k_iters = cdiv(pr.k, v.bk);
   const int occ = variant_occupancy(v, hw);
-  const double bkb = v.bk * esz;
+  const int area = v.bm * v.bn;
 
-  // per K step of one workgroup, in CU cycles (MFMA pipe and fill path are shared by the CU)
-  const double t_mfma = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type) / mfma_side_efficiency(v);
-  const double t_fill = (v.bm + v.bn) * bkb / (occ >= 2 ? 30.0 : 16.0);
-  const double t_iter = std::max(t_mfma, t_fill) + 60.0;
-  const double c_bytes = type_bits(pr.c_type) / 8.0;
-  const double t_epi = 2500.0 + v.bm * v.bn * c_bytes / 32.0;
+  const double ideal_step_us = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type) / clk * 1e6;
+  const double t_thru = ideal_step_us / family_efficiency(pr.a_type, v);   // CU time per tile K step, saturated
+  const double t_lat = 0.30 + (v.bm + v.bn) * (v.bk * esz) / 1.0e5;          // floor per K step of one workgroup: round trip + its own copy at ~100 GB/s
+  const double t_tile = area >= 256 * 256 ? 12.0 : (area >= 128 * 128 ? 4.0 : 3.0);
 
-  double cycles;
+  double us;
   if (streamk) {
     // K iterations spread evenly over every resident workgroup slot; one partial-tile fixup each
     const double slots = (double)hw.n_cu * occ;
-    const double iters_per_cu = std::ceil((double)tiles * k_iters / slots) * occ;
-    cycles = iters_per_cu * t_iter + t_epi * std::max(1.0, (double)tiles / slots) + 6000.0;
+    const double iters_per_slot = std::ceil((double)tiles * k_iters / slots);
+    us = iters_per_slot * std::max(occ * t_thru, t_lat) + t_tile * std::max(1.0, (double)tiles / slots) + 2.5;
   } else {
-    const double rounds = std::ceil((double)tiles / (double)hw.n_cu);  // tiles one CU works through
-    cycles = rounds * (k_iters * t_iter + t_epi / occ);
-    // a partly filled last round leaves CUs idle; small grids cannot use the L2-hit fill rate either
-    if (tiles < hw.n_cu) cycles = k_iters * t_iter + t_epi;
+    // the busiest CU works through c tiles, occ at a time
+    const int64_t c = cdiv(tiles, hw.n_cu);
+    const int64_t full = c / occ, rem = c % occ;
+    us = (double)full * (k_iters * std::max(occ * t_thru, t_lat) + t_tile);
+    if (rem) us += k_iters * std::max((double)rem * t_thru, t_lat) + t_tile;
   }
-  *comp_us = cycles / clk * 1e6;
+  *comp_us = us;
 
-  // HBM: every operand once, plus re-reads when a band of tiles does not stay in L2/MALL
+  // HBM: every operand once
+  const double c_bytes = type_bits(pr.c_type) / 8.0;
   const double a_bytes = (double)pr.m * pr.k * esz, b_bytes = (double)pr.n * pr.k * esz * std::max(1, pr.num_groups);
   const double c_out = (double)pr.m * pr.n * c_bytes;
   // few workgroups cannot pull the full HBM rate: ~45 GB/s per busy CU
