@@ -248,6 +248,8 @@ struct Operand {
   // compiler must not know that these vector-memory operations write LDS, otherwise it drains every
   // outstanding copy (vmcnt(0)) in front of the next LDS read and the software pipeline collapses.
   // Completion is tracked by hand with s_waitcnt vmcnt(N) before the barrier that publishes a stage.
+  // s_nop 3: one wait state between the write of m0 and its use, and five between a scalar base that
+  // the compiler may just have written with a vector instruction and the load that reads it.
   __device__ static __forceinline__ void dma(const St& st, int it, uint8_t* lds, int tid) {
     const uint8_t* gp = step_ptr(st, it);
     const int wave_slot = __builtin_amdgcn_readfirstlane(tid & ~63);
@@ -256,7 +258,7 @@ struct Operand {
     for (int i = 0; i < NCH; ++i) {
       if (CHUNKS % T::THREADS != 0 && i * T::THREADS + wave_slot >= CHUNKS) continue;
       const uint32_t dst = lds0 + (uint32_t)((i * T::THREADS + wave_slot) * 16);
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
                    : "s"(dst), "v"(st.off[i]), "s"(gp)
                    : "memory", "m0");
@@ -1000,25 +1002,60 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc,
 }
 
 // ------------------------------------------------------------------------------------------------
-// Stream-K partial tiles: fragment-ordered fp32 in P[slot], one float4 per lane per MFMA tile
+// Stream-K partial tiles: fragment-ordered fp32 in P[slot], one float4 per lane per MFMA tile.
+//
+// Publisher and owner usually sit on different XCDs, whose L2s are not coherent with each other for
+// ordinary accesses.  An acquire at device scope makes them so by invalidating the XCD's whole L2,
+// which throws away the operand lines every other workgroup of that XCD is working from -- and a
+// polling loop would do that on every poll.  So the partials and the flags move with device-scope
+// accesses (sc1, as relaxed device-scope atomics use): the stores write through, the loads bypass
+// stale lines and need no invalidate.  The publisher orders its stores before its flag with one release fence (the
+// reference: .wt stores, .cv loads, an atomic exchange as the release, streamk_gemm.py:196-262).
 // ------------------------------------------------------------------------------------------------
+// Both loops are assembly with a moving scalar base and one fixed 32-bit lane offset: 32 precomputed
+// 64-bit addresses next to 128 live accumulators would spill, and every reload of a spilled address
+// waits for all earlier write-through stores (vmcnt is shared), which serialises them.  The s_nop in
+// front of each access is required: the compiler may hand the base over in scalar registers it has
+// just written with a vector instruction (v_readlane from a spill slot), the hardware wants five wait
+// states between such a write and a vector-memory instruction that reads the register, and the
+// compiler's hazard pass does not look inside assembly statements.
 template <class T>
 __device__ __forceinline__ void partial_store(float* slot, v4f (&acc)[T::TM][T::TN], int tid) {
-#pragma unroll
-  for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j) *(v4f*)(slot + ((size_t)((i * T::TN + j) * T::THREADS + tid) << 2)) = acc[i][j];
-}
-
-template <class T>
-__device__ __forceinline__ void partial_add(const float* slot, v4f (&acc)[T::TM][T::TN], int tid) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t off = (uint32_t)tid * 16u;
 #pragma unroll
   for (int i = 0; i < T::TM; ++i)
 #pragma unroll
     for (int j = 0; j < T::TN; ++j) {
-      v4f v = *(const v4f*)(slot + ((size_t)((i * T::TN + j) * T::THREADS + tid) << 2));
-      acc[i][j] += v;
+      const float* base = slot + (size_t)(i * T::TN + j) * T::THREADS * 4;   // the scalar base moves, the lane offset stays
+      asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 sc1" : : "v"(off), "v"(acc[i][j]), "s"(base) : "memory");
     }
+#endif
+}
+
+template <class T>
+__device__ __forceinline__ void partial_add(const float* slot, v4f (&acc)[T::TM][T::TN], int tid) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NT = T::TM * T::TN;
+  constexpr int BATCH = (NT % 4 == 0) ? 4 : 1;
+  const uint32_t off = (uint32_t)tid * 16u;
+#pragma unroll
+  for (int t0 = 0; t0 < NT; t0 += BATCH) {
+    v4f v[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const float* base = slot + (size_t)(t0 + b) * T::THREADS * 4;
+      asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 sc1" : "=v"(v[b]) : "v"(off), "s"(base) : "memory");
+    }
+    // the compiler does not know that these registers are written asynchronously
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      asm volatile("" : "+v"(v[b]));
+      acc[(t0 + b) / T::TN][(t0 + b) % T::TN] += v[b];
+    }
+  }
+#endif
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1173,12 +1210,22 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
     __syncthreads();  // the previous item's store staging may still be read by slower waves
     mainloop<T, !SK>(p, w.tc, w.it0, w.it1, acc, lds, li);
     if constexpr (SK) {
+    if (w.kind == WK_FULL) {
+      // whole tiles get their own copy of the epilogue: sharing the one behind the fixup code makes
+      // the compiler park the accumulators in scratch on this, the common, path too
+      epilogue<T>(p, w.tc, acc, li, lds);
+      continue;
+    }
     if (w.kind == WK_SK_PUBLISH) {
       // not the tile's first segment: publish the partial, tagged with this launch's epoch
       partial_store<T>(p.P + (size_t)sched.pid * (T::BM * T::BN), acc, li.tid);
-      __threadfence();
-      __syncthreads();
-      if (li.tid == 0) __hip_atomic_store(p.flags + sched.pid, p.epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0x0070);   // this wave's write-through stores have left the CU
+      __syncthreads();                      // ... and so have everybody else's
+      if (li.tid == 0) {
+        // one L2 write-back for the workgroup (it covers every wave's stores), then the flag
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __hip_atomic_store(p.flags + sched.pid, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       continue;
     }
     if (w.kind == WK_SK_OWNER) {
@@ -1189,7 +1236,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
         if (li.tid == 0) {
           uint32_t spins = 0;
           int ok = 1;
-          while (__hip_atomic_load(p.flags + nxt, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
+          while (__hip_atomic_load(p.flags + nxt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
             if (++spins >= p.spin_limit) { ok = 0; break; }
             __builtin_amdgcn_s_sleep(2);
           }
@@ -1199,7 +1246,6 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
         int ok = s_bcast;
         __syncthreads();
         if (!ok) { failed = true; break; }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         partial_add<T>(p.P + (size_t)nxt * (T::BM * T::BN), acc, li.tid);
         cur_end += sched.q + (nxt < sched.rem ? 1 : 0);
         ++nxt;

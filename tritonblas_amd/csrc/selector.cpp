@@ -72,6 +72,19 @@ static double family_efficiency(int dt, const TileInfo& v) {
   return h16[cls];
 }
 
+// Stream-K launch grid for `total` tiles of `k_iters` K steps on `slots` co-resident workgroups.
+//   * fewer tiles than slots: every tile is cut into the same number s of K segments (grid = total * s),
+//     as many as fit the slots but never shorter than 16 K steps -- below that the fixup (one partial
+//     tile written, polled for and added per extra segment) costs more than the split saves;
+//   * otherwise every slot takes part: whole tiles first, the last total % slots tiles are shared.
+int streamk_grid(int64_t total, int64_t k_iters, int slots) {
+  if (total <= 0 || slots <= 0) return 1;
+  if (total >= slots) return slots;
+  int64_t s = std::max<int64_t>(1, slots / total);
+  s = std::min<int64_t>(s, std::max<int64_t>(1, k_iters / 16));
+  return (int)(total * s);
+}
+
 static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk, double* comp_us,
                     double* mem_us) {
   const double clk = hw.clock_khz * 1e3;
@@ -90,10 +103,20 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
 
   double us;
   if (streamk) {
-    // K iterations spread evenly over every resident workgroup slot; one partial-tile fixup each
-    const double slots = (double)hw.n_cu * occ;
-    const double iters_per_slot = std::ceil((double)tiles * k_iters / slots);
-    us = iters_per_slot * std::max(occ * t_thru, t_lat) + t_tile * std::max(1.0, (double)tiles / slots) + 2.5;
+    // one extra K segment of a tile costs its partial tile written through, polled for and added by the
+    // owner, one after the other: ~2 us + the fp32 tile at ~50 GB/s
+    const double fix_us = 2.0 + area * 4.0 / 50e3;
+    const int slots = hw.n_cu * occ;
+    const int grid = streamk_grid(tiles, k_iters, slots);
+    const double w = (double)cdiv(grid, hw.n_cu);                 // workgroups sharing the busiest CU
+    const double t_step = std::max(w * t_thru, t_lat);
+    const int64_t dp_rounds = tiles / grid, tail = tiles % grid;
+    us = (double)dp_rounds * (k_iters * t_step + t_tile);
+    if (tail > 0) {
+      const double iters = std::ceil((double)tail * k_iters / grid);
+      const double segments = std::ceil((double)grid / tail);
+      us += iters * t_step + (segments - 1.0) * fix_us + t_tile;
+    }
   } else {
     // the busiest CU works through c tiles, occ at a time
     const int64_t c = cdiv(tiles, hw.n_cu);
@@ -152,12 +175,7 @@ int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, in
   out->num_stages = v.stages;
   out->lds_bytes = v.lds_bytes;
   out->counters_per_xcd = ws_counters_per_xcd(total);
-  // Stream-K grid: every resident workgroup slot, but never more workgroups than K iterations to share
-  const int64_t k_iters = cdiv(pr.k, v.bk);
-  int64_t grid = (int64_t)hw.n_cu * out->occupancy;
-  grid = std::min(grid, total * k_iters);
-  if (total % grid == 0 && total >= grid) grid = std::min<int64_t>(grid, total);
-  out->sk_grid = (int)std::max<int64_t>(1, grid);
+  out->sk_grid = streamk_grid(total, cdiv(pr.k, v.bk), hw.n_cu * out->occupancy);
   out->est_compute_us = best_c; out->est_memory_us = best_m; out->est_total_us = best_t;
   return TB_OK;
 }

@@ -10,6 +10,7 @@ struct TileInfo {
 };
 
 void default_hw(tb_hw* hw);
+int streamk_grid(int64_t total_tiles, int64_t k_iters, int slots);
 int ws_counters_per_xcd(int64_t total_tiles);
 int variant_occupancy(const TileInfo& v, const tb_hw& hw);
 int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out);

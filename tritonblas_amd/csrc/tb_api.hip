@@ -286,13 +286,18 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     plan->ws_need = plan->ws_counters_off + (size_t)p.num_xcds * p.counters_per_xcd * COUNTER_STRIDE * 4;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
-    int64_t g = j.grid > 0 ? j.grid : std::min<int64_t>(resident, total * p.k_iters);
+    int64_t g = j.grid > 0 ? j.grid : streamk_grid(total, p.k_iters, resident);
     if (g > resident) return TB_ERR_BAD_SCHEDULE;  // owners spin on later workgroups: all must be resident
     grid = (int)g;
     p.sk_tiles = (int32_t)(total % grid);
-    plan->ws_flags_off = CTL_WORDS * 4;
-    plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
-    plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
+    if (p.sk_tiles == 0) {
+      // nothing to share: the same tiles on the whole-tile kernel (identical results, no workspace)
+      p.mode = MODE_STATIC;
+    } else {
+      plan->ws_flags_off = CTL_WORDS * 4;
+      plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
+      plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
+    }
   } else {
     return TB_ERR_BAD_SCHEDULE;
   }
