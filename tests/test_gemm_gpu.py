@@ -199,6 +199,30 @@ def test_streamk_explicit_grid(m, n, k, grid, dtype):
         _check(c.cpu(), want, dtype, TOL_16)
 
 
+@pytest.mark.parametrize("m,n,k,grid", [(512, 512, 4096, 64), (300, 700, 8192, 200), (256, 256, 16384, 256)])
+def test_streamk_workspace_reuse_with_new_data(m, n, k, grid):
+    """Back-to-back Stream-K launches on ONE workspace with different operands each time: a partial tile
+    or flag left behind by an earlier launch (in the workspace or in any cache on the way) must never
+    reach a later result.  No synchronisation between the launches."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    _say(f"stream-k workspace reuse {m}x{n}x{k} grid={grid}")
+    dtype = torch.bfloat16
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, torch.device("cuda", 0), streamk=True)
+    cfg = tb.matmul_preamble(sel)
+    cases = []
+    for rep in range(5):
+        a_cpu, b_cpu = _rand((m, k), dtype, 100 + rep, 0.5), _rand((k, n), dtype, 200 + rep, 0.5)
+        cases.append((a_cpu, b_cpu, a_cpu.cuda(), b_cpu.cuda(), torch.zeros(m, n, dtype=dtype, device="cuda")))
+    torch.cuda.synchronize()
+    for (_, _, a, b, c) in cases:
+        streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=grid)
+    torch.cuda.synchronize()
+    assert cfg.status() == 0
+    for rep, (a_cpu, b_cpu, _, _, c) in enumerate(cases):
+        _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32), dtype, TOL_16)
+
+
 @pytest.mark.parametrize("kernel", ["streaming", "streamk"])
 def test_decode_shape_small(kernel, monkeypatch):
     """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly:
