@@ -202,3 +202,30 @@ def test_default_panel_is_a_near_square_multiple_of_the_xcd_block():
     assert lib.tb_default_panel(512, 64, 8) == 24
     assert lib.tb_default_panel(1, 1, 1) == 1
     assert lib.tb_default_panel(7, 1, 8) == 3
+
+
+# ---- torch custom operators: registration and shape rules (no GPU needed) -------------------------
+def test_custom_ops_are_registered_with_the_reference_signatures():
+    import tritonblas_amd  # noqa: F401  (registers the operators)
+    ops = torch.ops.tritonblas_amd
+    assert str(ops._matmul.default._schema) == ("tritonblas_amd::_matmul(Tensor a, Tensor b, bool? enable_streamk=False, "
+                                                "SymInt? sk_grid=None, bool? work_stealing=False) -> Tensor")
+    assert "Tensor(a2!) out" in str(ops._matmul_out.default._schema) and str(ops._matmul_out.default._schema).endswith("-> ()")
+    assert str(ops._addmm.default._schema).startswith("tritonblas_amd::_addmm(Tensor bias, Tensor a, Tensor b,")
+    assert "Tensor(a3!) out" in str(ops._addmm_out.default._schema)
+
+
+def test_custom_op_fake_implementations_propagate_shapes():
+    import tritonblas_amd as tb
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        a = torch.empty(64, 32, device="cuda", dtype=torch.bfloat16)
+        b = torch.empty(32, 48, device="cuda", dtype=torch.bfloat16)
+        bias = torch.empty(48, device="cuda", dtype=torch.bfloat16)
+        c = tb.matmul(a, b)
+        assert tuple(c.shape) == (64, 48) and c.dtype == torch.bfloat16 and c.device.type == "cuda"
+        assert tuple(tb.addmm(bias, a, b, enable_streamk=True).shape) == (64, 48)
+        out = torch.empty(64, 48, device="cuda", dtype=torch.bfloat16)
+        assert tb.matmul(a, b, out=out) is None and tb.addmm(bias, a, b, out=out) is None
+        with pytest.raises(Exception, match="Incompatible A-B Dimensions"):
+            tb.matmul(a, torch.empty(31, 48, device="cuda", dtype=torch.bfloat16))

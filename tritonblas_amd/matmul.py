@@ -135,48 +135,106 @@ def _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, out_dtype_for_
     return persistent_matmul_lt(a, b, out, selector, config, bias=bias, work_stealing=work_stealing)
 
 
-class _MatmulFn(torch.autograd.Function):
-    """Forward through the library, backward as two more library GEMMs (reference matmul.py:393-448)."""
-
-    @staticmethod
-    def forward(ctx, a, b, enable_streamk, sk_grid, work_stealing):
-        assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
-        out = a.new_empty(a.shape[0], b.shape[1])
-        _run(a.detach(), b.detach(), out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
-        ctx.save_for_backward(a, b)
-        ctx.opts = (enable_streamk, sk_grid, work_stealing)
-        return out
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        a, b = ctx.saved_tensors
-        sk, grid, ws = ctx.opts
-        g = grad_output.contiguous()
-        grad_a = matmul(g, b.detach().T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
-        grad_b = matmul(a.detach().T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
-        return grad_a, grad_b, None, None, None
+# ---- torch custom operators (reference matmul.py:393-472, 628-752) ----------------------------------
+# Registered with torch.library so that autograd and torch.compile (fullgraph) see one opaque operator
+# with a shape rule (fake implementation) instead of a ctypes call they cannot trace.  The reference
+# registers the same four operators with triton_op; the namespace differs so that both packages can be
+# imported side by side.
+def _fake_new_output(a, b):
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    return a.new_empty(a.shape[0], b.shape[1])
 
 
-class _AddmmFn(torch.autograd.Function):
-    """Reference matmul.py:628-696."""
+@torch.library.custom_op("tritonblas_amd::_matmul", mutates_args=())
+def _matmul(a: torch.Tensor, b: torch.Tensor, enable_streamk: Optional[bool] = False, sk_grid: Optional[int] = None,
+            work_stealing: Optional[bool] = False) -> torch.Tensor:
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    out = a.new_empty(a.shape[0], b.shape[1])
+    _run(a, b, out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
+    return out
 
-    @staticmethod
-    def forward(ctx, bias, a, b, enable_streamk, sk_grid, work_stealing):
-        assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
-        out = a.new_empty(a.shape[0], b.shape[1])
-        _run(a.detach(), b.detach(), out, bias.detach(), enable_streamk, sk_grid, work_stealing, bias.dtype)
-        ctx.save_for_backward(a, b)
-        ctx.opts = (enable_streamk, sk_grid, work_stealing)
-        return out
 
-    @staticmethod
-    def backward(ctx, grad_output):
-        a, b = ctx.saved_tensors
-        sk, grid, ws = ctx.opts
-        g = grad_output.contiguous()
-        grad_a = matmul(g, b.detach().T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
-        grad_b = matmul(a.detach().T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
-        return grad_output.sum(dim=0), grad_a, grad_b, None, None, None
+@_matmul.register_fake
+def _(a, b, enable_streamk=False, sk_grid=None, work_stealing=False):
+    return _fake_new_output(a, b)
+
+
+def _matmul_setup_context(ctx, inputs, output):
+    a, b, enable_streamk, sk_grid, work_stealing = inputs
+    ctx.save_for_backward(a, b)
+    ctx.opts = (enable_streamk, sk_grid, work_stealing)
+
+
+def _matmul_backward(ctx, grad_output):
+    # two more library GEMMs: grad_a = g @ b^T, grad_b = a^T @ g
+    a, b = ctx.saved_tensors
+    sk, grid, ws = ctx.opts
+    g = grad_output.contiguous()
+    grad_a = matmul(g, b.T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+    grad_b = matmul(a.T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+    return grad_a, grad_b, None, None, None
+
+
+_matmul.register_autograd(_matmul_backward, setup_context=_matmul_setup_context)
+
+
+@torch.library.custom_op("tritonblas_amd::_matmul_out", mutates_args={"out"})
+def _matmul_out(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, enable_streamk: Optional[bool] = False,
+                sk_grid: Optional[int] = None, work_stealing: Optional[bool] = False) -> None:
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    _run(a, b, out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
+
+
+@_matmul_out.register_fake
+def _(a, b, out, enable_streamk=False, sk_grid=None, work_stealing=False):
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    return None
+
+
+@torch.library.custom_op("tritonblas_amd::_addmm", mutates_args=())
+def _addmm(bias: torch.Tensor, a: torch.Tensor, b: torch.Tensor, enable_streamk: Optional[bool] = False,
+           sk_grid: Optional[int] = None, work_stealing: Optional[bool] = False) -> torch.Tensor:
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    out = a.new_empty(a.shape[0], b.shape[1])
+    _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, bias.dtype)
+    return out
+
+
+@_addmm.register_fake
+def _(bias, a, b, enable_streamk=False, sk_grid=None, work_stealing=False):
+    return _fake_new_output(a, b)
+
+
+def _addmm_setup_context(ctx, inputs, output):
+    bias, a, b, enable_streamk, sk_grid, work_stealing = inputs
+    ctx.save_for_backward(a, b)
+    ctx.opts = (enable_streamk, sk_grid, work_stealing)
+
+
+def _addmm_backward(ctx, grad_output):
+    a, b = ctx.saved_tensors
+    sk, grid, ws = ctx.opts
+    g = grad_output.contiguous()
+    grad_a = matmul(g, b.T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+    grad_b = matmul(a.T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
+    return grad_output.sum(dim=0), grad_a, grad_b, None, None, None
+
+
+_addmm.register_autograd(_addmm_backward, setup_context=_addmm_setup_context)
+
+
+@torch.library.custom_op("tritonblas_amd::_addmm_out", mutates_args={"out"})
+def _addmm_out(bias: torch.Tensor, a: torch.Tensor, b: torch.Tensor, out: torch.Tensor,
+               enable_streamk: Optional[bool] = False, sk_grid: Optional[int] = None,
+               work_stealing: Optional[bool] = False) -> None:
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, bias.dtype)
+
+
+@_addmm_out.register_fake
+def _(bias, a, b, out, enable_streamk=False, sk_grid=None, work_stealing=False):
+    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
+    return None
 
 
 def matmul(a, b, out: Optional[torch.Tensor] = None, enable_streamk: Optional[bool] = False,
@@ -184,30 +242,26 @@ def matmul(a, b, out: Optional[torch.Tensor] = None, enable_streamk: Optional[bo
     """Reference matmul.py:475-495: out=None allocates and supports autograd; out=... writes in
     place, returns None and refuses tensors that require grad."""
     if out is None:
-        return _MatmulFn.apply(a, b, enable_streamk, sk_grid, work_stealing)
+        return _matmul(a, b, enable_streamk, sk_grid, work_stealing)
     if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad or out.requires_grad):
         raise RuntimeError(
             "tritonblas.matmul(): functions with out=... arguments don't support "
             "automatic differentiation, but one of the arguments requires grad."
         )
-    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
-    _run(a, b, out, None, enable_streamk, sk_grid, work_stealing, out.dtype)
-    return None
+    return _matmul_out(a, b, out, enable_streamk, sk_grid, work_stealing)
 
 
 def addmm(bias, a, b, out: Optional[torch.Tensor] = None, enable_streamk: Optional[bool] = False,
           sk_grid: Optional[int] = None, work_stealing: Optional[bool] = False) -> Optional[torch.Tensor]:
     """Reference matmul.py:727-752; the bias is added per output column."""
     if out is None:
-        return _AddmmFn.apply(bias, a, b, enable_streamk, sk_grid, work_stealing)
+        return _addmm(bias, a, b, enable_streamk, sk_grid, work_stealing)
     if torch.is_grad_enabled() and (bias.requires_grad or a.requires_grad or b.requires_grad or out.requires_grad):
         raise RuntimeError(
             "tritonblas.addmm(): functions with out=... arguments don't support "
             "automatic differentiation, but one of the arguments requires grad."
         )
-    assert a.shape[1] == b.shape[0], "Incompatible A-B Dimensions"
-    _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, bias.dtype)
-    return None
+    return _addmm_out(bias, a, b, out, enable_streamk, sk_grid, work_stealing)
 
 
 def matmul_a8w8(a, b, a_scale, b_scale, c, enable_streamk=False, work_stealing=False, sk_grid=None):
