@@ -1,0 +1,59 @@
+"""Benchmark driver (YAML shape list -> CSV): column set and flags of the reference's
+benchmarks/tritonblas_matmul.py; shape lists of datasets/generate_grid*.py."""
+import csv
+
+import pytest
+import yaml
+
+REFERENCE_COLUMNS = ["m", "n", "k", "mnk", "macro_tile", "bytes", "flops", "tritonblas_gflops", "a_type", "b_type", "c_type",
+                     "d_type", "compute_type", "in_dtype", "out_dtype", "init_type", "transA", "transB", "us", "alpha", "beta",
+                     "mode"]   # benchmarks/tritonblas_matmul.py:287-293
+
+
+def test_csv_columns_are_the_reference_ones():
+    from tritonblas_amd.benchmarks import matmul_bench
+    assert matmul_bench.FIELDNAMES == REFERENCE_COLUMNS
+
+
+def test_generate_grid_presets(tmp_path):
+    from tritonblas_amd.benchmarks import generate_grid
+    out = tmp_path / "g.yaml"
+    generate_grid.main(["--preset", "grid", "--min", "1024", "--max", "2048", "--step", "1024", "-o", str(out)])
+    cases = yaml.safe_load(out.read_text())
+    assert len(cases) == 8 and cases[0] == {"m": 1024, "n": 1024, "k": 1024, "in_dtype": "float16", "out_dtype": "float16",
+                                            "transA": "T", "transB": "N"}
+    generate_grid.main(["--preset", "fp4", "--out-dtype", "bfloat16", "-o", str(out)])
+    cases = yaml.safe_load(out.read_text())
+    assert len(cases) == 19 and all(c["in_dtype"] == "fp4" and c["k"] % 32 == 0 for c in cases)   # generate_grid_fp4.py:12-36
+    assert (cases[0]["m"], cases[0]["n"], cases[0]["k"]) == (256, 2048, 8192)
+
+
+def test_dtype_names():
+    import torch
+    from tritonblas_amd.benchmarks.matmul_bench import str_to_dtype
+    assert str_to_dtype("bfloat16") is torch.bfloat16 and str_to_dtype("torch.float8_e4m3fn") is torch.float8_e4m3fn
+    assert str_to_dtype("fp4") == "fp4"
+    with pytest.raises(ValueError):
+        str_to_dtype("int8")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("flags", [[], ["--enable-streamk"], ["--work-stealing"]])
+def test_driver_runs_a_shape_list_with_correctness_check(tmp_path, flags):
+    from tritonblas_amd.benchmarks import matmul_bench
+    print(f"bench driver {flags}", flush=True)
+    cases = [
+        {"m": 256, "n": 512, "k": 1024, "in_dtype": "bfloat16", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+        {"m": 300, "n": 200, "k": 512, "in_dtype": "float16", "out_dtype": "float16", "transA": "T", "transB": "T"},
+        {"m": 512, "n": 256, "k": 2048, "in_dtype": "float8_e4m3fn", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+    ]
+    if not flags:
+        cases.append({"m": 128, "n": 256, "k": 1024, "in_dtype": "fp4", "out_dtype": "bfloat16", "transA": "T", "transB": "N"})
+    src, dst = tmp_path / "shapes.yaml", tmp_path / "out.csv"
+    src.write_text(yaml.safe_dump(cases))
+    matmul_bench.main(["--input-yaml", str(src), "--output-csv", str(dst), "--checkcorrectness", "--n-warmup", "2",
+                       "--n-repeat", "3"] + flags)
+    rows = list(csv.DictReader(dst.open()))
+    assert len(rows) == len(cases) and list(rows[0].keys()) == REFERENCE_COLUMNS
+    want_mode = "work_stealing" if "--work-stealing" in flags else ("streamk" if "--enable-streamk" in flags else "persistent")
+    assert all(r["mode"] == want_mode and float(r["tritonblas_gflops"]) > 0 for r in rows)
