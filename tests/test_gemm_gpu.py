@@ -243,12 +243,13 @@ def test_decode_shape_small(kernel, monkeypatch):
     assert cfg.status() == 0
 
 
-@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("m,n,k", [(m, 1040, 2304) for m in (1, 5, 16, 17, 32, 33, 64)] +
+                         [(m, 24576 + 40, 256) for m in (7, 32, 64)])   # wide N: 64-column workgroups
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
-def test_skinny_rows(m, dtype):
-    """Every row-block count of the streaming kernel, ragged N, bias, all three element types."""
+def test_skinny_rows(m, n, k, dtype):
+    """Every row-block count of the streaming kernel and both column widths of its workgroups, ragged N,
+    bias, all three element types."""
     import tritonblas_amd as tb
-    n, k = 1040, 2304
     _say(f"skinny {m}x{n}x{k} {dtype}")
     if dtype == torch.float8_e4m3fn:
         aq, bq, sa, sb = _a8w8_case(m, n, k, seed=31)

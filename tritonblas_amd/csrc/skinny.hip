@@ -121,17 +121,21 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(const GemmParams p) 
   }
 }
 
-template <int DT, int MT>
-static hipError_t launch_mt(const GemmParams& p, hipStream_t stream) {
-#ifndef SK_NT
-#define SK_NT 2
-#define SK_WAVES 8
-#define SK_DEPTH 4
-#endif
-  constexpr int NT = SK_NT, WAVES = SK_WAVES, DEPTH = SK_DEPTH;
+template <int DT, int MT, int NT, int DEPTH>
+static hipError_t launch_nt(const GemmParams& p, hipStream_t stream) {
+  constexpr int WAVES = 8;
   const int grid = (p.N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((skinny_kernel<DT, MT, NT, WAVES, DEPTH>), dim3(grid), dim3(WAVES * 64), 0, stream, p);
   return hipGetLastError();
+}
+
+// Every workgroup reads all of A (from L2), so its cost per weight byte halves when a workgroup owns
+// 64 columns instead of 32 -- worth it once 64-column workgroups still outnumber the CUs well
+// (measured on 256 CUs: N = 28672, K = 8192, M = 32: 70 us -> 48 us; N = 8192 would leave half the CUs idle).
+template <int DT, int MT>
+static hipError_t launch_mt(const GemmParams& p, hipStream_t stream) {
+  if (p.N >= 64 * 384) return launch_nt<DT, MT, 4, 2>(p, stream);
+  return launch_nt<DT, MT, 2, 4>(p, stream);
 }
 
 template <int DT>
