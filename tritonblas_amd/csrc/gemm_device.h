@@ -1138,29 +1138,50 @@ struct Sched {
     }
     if (p.mode == MODE_WS) {
       // Queues: one counter per (xcd, slot).  A workgroup drains its own queue, then the other
-      // slots of its XCD, then the other XCDs' queues.
+      // slots of its XCD, then the other XCDs' queues.  Visit number `step` is queue
+      // ((xcd + step / S) % X, (slot + step % S) % S).  The first wave looks at 64 visits at a time:
+      // every lane reads one queue's counter, the first queue (in visiting order) that still has
+      // tiles gets the atomic increment, and if somebody else emptied it meanwhile the next one is
+      // tried.  One round trip finds the next tile -- or finds that everything is gone -- instead of
+      // one per queue.
       const int X = p.num_xcds, S = p.counters_per_xcd;
       const int xcd = pid % X, slot = (pid / X) % S;
       const int per_xcd = (p.total_tiles + X - 1) / X;
-      while (step < X * S) {
-        int qx = (xcd + step / S) % X;
-        int qs = (slot + step % S) % S;
-        int xbase = qx * per_xcd;
-        int xcnt = max(min(xbase + per_xcd, p.total_tiles) - xbase, 0);
-        int per_slot = (xcnt + S - 1) / S;
-        int sbase = qs * per_slot;
-        int bound = max(min(sbase + per_slot, xcnt) - sbase, 0);
-        if (tid == 0) *s_bcast = (bound > 0) ? atomicAdd(p.counters + (qx * S + qs) * COUNTER_STRIDE, 1) : 0;
-        __syncthreads();
-        int idx = *s_bcast;
-        __syncthreads();
-        if (idx < bound) {
-          plain_tile(p, xbase + sbase + idx, T::BM, T::BN, w.tc);
-          return true;
+      if (tid < 64) {
+        const int lane = tid;
+        int found = -1, found_step = X * S;
+        for (int base = step; base < X * S && found < 0; base += 64) {
+          const int v = base + lane;
+          const bool valid = v < X * S;
+          const int qx = (xcd + v / S) % X;
+          const int qs = (slot + v % S) % S;
+          const int xbase = qx * per_xcd;
+          const int xcnt = max(min(xbase + per_xcd, p.total_tiles) - xbase, 0);
+          const int per_slot = (xcnt + S - 1) / S;
+          const int sbase = qs * per_slot;
+          const int bound = valid ? max(min(sbase + per_slot, xcnt) - sbase, 0) : 0;
+          int32_t* ctr = p.counters + (qx * S + qs) * COUNTER_STRIDE;
+          const int seen = bound > 0 ? __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+          unsigned long long open = __ballot(bound > 0 && seen < bound);
+          while (open != 0 && found < 0) {
+            const int l = __builtin_ctzll(open);
+            int idx = 0;
+            if (lane == l) idx = atomicAdd(ctr, 1);
+            idx = __shfl(idx, l);
+            const int b = __shfl(bound, l), first = __shfl(xbase + sbase, l);
+            if (idx < b) { found = first + idx; found_step = base + l; }
+            open &= open - 1;
+          }
         }
-        ++step;
+        if (lane == 0) { s_bcast[0] = found; s_bcast[1] = found_step; }
       }
-      return false;
+      __syncthreads();
+      const int tile = s_bcast[0];
+      step = s_bcast[1];
+      __syncthreads();
+      if (tile < 0) return false;
+      plain_tile(p, tile, T::BM, T::BN, w.tc);
+      return true;
     }
     if constexpr (!SK) return false;
     // MODE_SK: data-parallel tiles first, then this workgroup's share of the Stream-K iterations
