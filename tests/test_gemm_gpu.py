@@ -308,6 +308,23 @@ def test_fp4_scale_extremes():
     _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.float32, 1e-5)
 
 
+@pytest.mark.parametrize("tile", [(256, 256, 256), (128, 128, 256), (128, 128, 128), (64, 64, 256)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (320, 448, 1536), (512, 256, 4096)])
+def test_fp4_fast_kernels_random_scales(tile, m, n, k):
+    """The LDS-direct kernels (K a multiple of 512) stage the scale bytes through LDS group by group:
+    random codes and random, widely varying scale bytes over several groups pin every byte's place."""
+    import tritonblas_amd as tb
+    _say(f"fp4 fast tile={tile} {m}x{n}x{k}")
+    rng = np.random.default_rng(m + k)
+    xq = torch.from_numpy(rng.integers(0, 256, (m, k // 2), dtype=np.uint8))
+    wq = torch.from_numpy(rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
+    xs = torch.from_numpy(rng.integers(100, 150, (m, k // 32), dtype=np.uint8))
+    ws = torch.from_numpy(rng.integers(100, 150, (n, k // 32), dtype=np.uint8))
+    c = torch.zeros(m, n, dtype=torch.float32, device="cuda")
+    tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda(), block_m=tile[0], block_n=tile[1], block_k=tile[2])
+    _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.float32, 1e-5)
+
+
 # ---- grouped MoE --------------------------------------------------------------------------------
 @pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [0, 0, 5]])
 def test_grouped_a8w8(counts):

@@ -99,11 +99,13 @@ struct Tile {
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-  // MX scales (fp4, LDS-direct kernels): 32 scale bytes per tile row are staged in LDS at a time,
-  // i.e. the scales of SCG consecutive K steps (one 32-element block = one 16-byte chunk = one byte).
-  static constexpr int SC_GB = 32;
+  // MX scales (fp4, LDS-direct kernels): 16 scale bytes per tile row are staged in LDS at a time,
+  // i.e. the scales of SCG consecutive K steps (one 32-element block = one 16-byte chunk = one byte),
+  // in two buffers: one is read while the other takes the next group.
+  static constexpr int SC_GB = 16;
   static constexpr int SCG = (DT == DT_FP4) ? SC_GB / CPR : 1;
-  static constexpr int SC_BYTES = (DT == DT_FP4 && DMA) ? (BM + BN) * SC_GB : 0;
+  static constexpr int SC_BUF = (BM + BN) * SC_GB;
+  static constexpr int SC_BYTES = (DT == DT_FP4 && DMA) ? 2 * SC_BUF : 0;
   static constexpr int LDS_TOTAL = LDS_BYTES + SC_BYTES;
   static constexpr int LDS_LIMIT = 160 * 1024;
   // the one word the schedules broadcast through LDS lives in the tile buffer's last 16 bytes when
@@ -400,8 +402,7 @@ __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70);
 // ------------------------------------------------------------------------------------------------
 // K loop: accumulates k iterations [it0, it1) of one output tile
 // ------------------------------------------------------------------------------------------------
-// WHOLE: the caller only ever passes complete tiles (it0 = 0, it1 = k_iters); lets the fp4 kernels
-// unroll the K loop over one scale group.
+// WHOLE: the caller only ever passes complete tiles (it0 = 0, it1 = k_iters).
 template <class T, bool WHOLE>
 __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc, int it0, int it1,
                                          v4f (&acc)[T::TM][T::TN], uint8_t* lds, const LaneInfo& li) {
@@ -441,22 +442,11 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     }
   };
 
-  // One K step of MFMAs from an LDS stage.  The A-side fragment of row block i+1 is requested before
-  // the MFMAs of row block i are issued, so an LDS read is always in flight under the matrix pipe.
-  // fp4 kernels with LDS-staged scales keep the scale bytes of the SCG K steps of a group in ga/gb
-  // (8 bytes per lane and row block: step s, slice ks at byte s*KSUB+ks).  With a compile-time step
-  // position SC >= 0 the byte is picked by register index and op_sel; SC = -1 uses sca/scb.
-  constexpr bool MXG = (T::DT == DT_FP4) && T::DMA;
-  uint32_t ga[T::TM][2], gb[T::TN][2];
-#pragma unroll
-  for (int i = 0; i < T::TM; ++i) ga[i][0] = ga[i][1] = 0;
-#pragma unroll
-  for (int j = 0; j < T::TN; ++j) gb[j][0] = gb[j][1] = 0;
+  constexpr bool MXG = (T::DT == DT_FP4) && T::DMA;   // MX scales staged through LDS
 
   // One K step of MFMAs from an LDS stage.  The A-side fragment of row block i+1 is requested before
   // the MFMAs of row block i are issued, so an LDS read is always in flight under the matrix pipe.
-  auto compute = [&](auto SC, const uint8_t* sA, const uint8_t* sB) {
-    constexpr int SCV = decltype(SC)::value;
+  auto compute = [&](const uint8_t* sA, const uint8_t* sB) {
 #pragma unroll
     for (int ks = 0; ks < T::KSUB; ++ks) {
       frag_t bf[T::TN];
@@ -471,13 +461,8 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         for (int j = 0; j < T::TN; ++j) {
           // output rows follow the first MFMA operand: feed B there so that one lane owns four
           // consecutive n of one m (contiguous in a row-major C).
-#define TB_MMA(KS)                                                                                             \
-  if (ks == KS) {                                                                                              \
-    constexpr bool ST = MXG && SCV >= 0;                                                                       \
-    constexpr int BYTE = ST ? (SCV * T::KSUB + KS) : KS;                                                       \
-    acc[i][j] = mma<T, (BYTE & 3)>(bf[j], af[i & 1], acc[i][j], ST ? gb[j][(BYTE >> 2) & 1] : scb[j],           \
-                                   ST ? ga[i][(BYTE >> 2) & 1] : sca[i]);                                       \
-  }
+#define TB_MMA(KS) \
+  if (ks == KS) acc[i][j] = mma<T, KS>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
           TB_MMA(0) TB_MMA(1) TB_MMA(2) TB_MMA(3)
 #undef TB_MMA
         }
@@ -495,13 +480,69 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     }
   };
 
-  if constexpr (T::DMA && !MXG) {
+  if constexpr (T::DMA) {
     constexpr int S = T::STAGES;
     // Stage (it - it0) % S holds K step `it`.  One "group" is what a wave issues per K step: its share
     // of both operand copies.  All S stages are filled up front; afterwards the copy of step it+S is
     // issued in the middle of step `it`, right after the barrier that frees that step's stage.
     constexpr int NG = OA::NCH + OB::NCH;
     static_assert((S - 1) * NG <= 63, "vmcnt range");
+
+    // ---- MX scales (fp4).  A scale group = SC_GB scale bytes of every tile row = the scales of SCG
+    // K steps; group g is copied raw into buffer g & 1: per row [step][lane group][KSUB bytes], so
+    // the KSUB bytes a lane needs for one K step and row block are one small LDS read, straight
+    // from the copy.  The scales of step it+1 are read during the last slice of step `it`: those of
+    // row block i once its MFMAs are issued, the rest behind the barrier.  Group g is therefore
+    // requested after the barrier of step g*SCG - 3 (everybody has then read the last scales of
+    // group g-2) and has landed by the wait of step g*SCG - 2, whose barrier publishes it (the
+    // scale copy is issued ahead of the operand copies of its step, and the wait of the next step
+    // lets at most one step's operand copies stay in flight).
+    uint8_t* sc_lds = lds + T::LDS_BYTES;
+    constexpr int NQ = T::BM + T::BN;                               // one 16-byte chunk per row and group
+    constexpr int NSCH = MXG ? (NQ + T::THREADS - 1) / T::THREADS : 1;
+    static_assert(!MXG || T::SC_GB == 16, "one copy chunk per row");
+    static_assert(!MXG || T::KSUB <= 2, "scale reads are one or two bytes");
+    constexpr int SC_LEAD = 3;
+    static_assert(!MXG || S <= 3, "with deeper pipelines the scale copy would land a step later");
+    static_assert(!MXG || T::SCG + 1 >= SC_LEAD, "a scale buffer is free again before its next group is requested");
+    const uint8_t* scp[NSCH];
+    const int g0 = it0 / T::SCG;
+    const uint8_t* sc_ra = sc_lds + (li.wm0 + li.r) * T::SC_GB + li.g * T::KSUB;
+    const uint8_t* sc_rb = sc_lds + (T::BM + li.wn0 + li.r) * T::SC_GB + li.g * T::KSUB;
+    if constexpr (MXG) {
+#pragma unroll
+      for (int i = 0; i < NSCH; ++i) {
+        const int row = i * T::THREADS + li.tid;
+        if (row < T::BM) scp[i] = p.mxa + (int64_t)min(tc.m0 + row, tc.m_lim - 1) * p.mxa_sr;
+        else scp[i] = p.mxb + (int64_t)min(tc.n0 + row - T::BM, tc.n_lim - 1) * p.mxb_sr;
+      }
+    }
+    auto sc_dma = [&](int grp) {
+      if constexpr (MXG) {
+        const int wave_slot = __builtin_amdgcn_readfirstlane(li.tid & ~63);
+        const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)sc_lds) + (grp & 1) * T::SC_BUF;
+#pragma unroll
+        for (int i = 0; i < NSCH; ++i) {
+          if (NQ % T::THREADS != 0 && i * T::THREADS + wave_slot >= NQ) continue;
+          const uint32_t dst = lds0 + (uint32_t)((i * T::THREADS + wave_slot) * 16);
+          const uint8_t* src = scp[i] + (int64_t)grp * T::SC_GB;
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
+        }
+      }
+    };
+    // the scale bytes of K step `it`: sca for q < TM, scb behind
+    auto sc_request = [&](int it, int q, uint32_t(&xa)[T::TM], uint32_t(&xb)[T::TN]) {
+      if constexpr (MXG) {
+        const int off = ((it / T::SCG) & 1) * T::SC_BUF + (it % T::SCG) * T::CPR;
+        const uint8_t* src = (q < T::TM) ? sc_ra + off + q * 16 * T::SC_GB : sc_rb + off + (q - T::TM) * 16 * T::SC_GB;
+        const uint32_t v = (T::KSUB == 2) ? (uint32_t)(*(const uint16_t*)src) : (uint32_t)(*src);
+        if (q < T::TM) xa[q] = v; else xb[q - T::TM] = v;
+      }
+    };
+    if constexpr (MXG) {
+      sc_dma(g0);
+      if ((g0 + 1) * T::SCG < it1) sc_dma(g0 + 1);
+    }
     int issued = 0;
 #pragma unroll
     for (int s = 0; s < S; ++s) {
@@ -515,6 +556,10 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     if (issued == S) __builtin_amdgcn_s_waitcnt(0x0F70 | (((S - 1) * NG) & 0xF) | ((((S - 1) * NG) >> 4) << 14));
     else wait_vm0();
     __syncthreads();
+    if constexpr (MXG) {
+#pragma unroll
+      for (int q = 0; q < T::TM + T::TN; ++q) sc_request(it0, q, sca, scb);
+    }
 
     // ---- software pipeline over (K step, MFMA slice) blocks ------------------------------------
     // On entry to a block its B fragments and its first A fragment are already in registers: they
@@ -533,20 +578,34 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     // afterwards the fragments of slice nks of stage (nA, nB) are requested.  After the last step of
     // the range that request still runs (no branch in the pipeline): it reads whatever the next stage
     // holds and nobody uses the result.
-    auto block = [&](auto KSC, const uint8_t* sA, auto&& boundary, const uint8_t* nA, const uint8_t* nB, int nks) {
+    auto block = [&](auto KSC, const uint8_t* sA, auto&& boundary, const uint8_t* nA, const uint8_t* nB, int nks, int nit) {
       constexpr int KSV = decltype(KSC)::value;
+      constexpr bool LAST = MXG && KSV + 1 == T::KSUB;   // the next block belongs to K step nit: fetch its scales
       frag_t af[2];
       af[0] = afn;
 #pragma unroll
       for (int i = 0; i < T::TM; ++i) {
+        if constexpr (LAST) { if (i >= 1) sc_request(nit, i - 1, nsca, nscb); }
         if (i + 1 < T::TM) af[(i + 1) & 1] = request_a(sA, KSV, i + 1);
         if (i + 1 == T::TM) {
           // pin the issue order so far for the machine scheduler (the barrier inside `boundary` ends
-          // a scheduling region): one fragment request, then one row block of MFMAs
+          // a scheduling region): one fragment request (plus a scale read), then one row block of MFMAs
 #pragma unroll
           for (int q = 0; q + 1 < T::TM; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+            if (LAST && q >= 1) __builtin_amdgcn_sched_group_barrier(0x100, RPF + 1, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, T::TN, 0);
+          }
+          if constexpr (LAST) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            // instruction selection is free to place the (side-effect-free) MFMAs behind the
+            // barrier; an empty statement that "uses" their results keeps them in front of it
+#pragma unroll
+            for (int q = 0; q + 1 < T::TM; ++q) {
+              static_assert(!MXG || T::TN == 4 || T::TN == 2, "pin list");
+              if constexpr (T::TN == 4) asm volatile("" : "+v"(acc[q][0]), "+v"(acc[q][1]), "+v"(acc[q][2]), "+v"(acc[q][3]));
+              else asm volatile("" : "+v"(acc[q][0]), "+v"(acc[q][1]));
+            }
           }
           boundary();
           afn = request_a(nA, nks, 0);
@@ -555,16 +614,35 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         for (int j = 0; j < T::TN; ++j) {
           // output rows follow the first MFMA operand: feed B there so that one lane owns four
           // consecutive n of one m (contiguous in a row-major C).
-          acc[i][j] = mma<T, 0>(bf[j], af[i & 1], acc[i][j], 0u, 0u);
-          if (i + 1 == T::TM) request_b(nB, nks, j);
+          acc[i][j] = mma<T, MXG ? KSV : 0>(bf[j], af[i & 1], acc[i][j], scb[j], sca[i]);
+          if (i + 1 == T::TM) {
+            request_b(nB, nks, j);
+            if constexpr (LAST) {
+              if (j == 0) sc_request(nit, T::TM - 1, nsca, nscb);
+              sc_request(nit, T::TM + j, nsca, nscb);
+            }
+          }
         }
       }
-      // last row block: the next A fragment, then MFMAs and B fragment requests alternate
+      // last row block: the next A fragment, then MFMAs and B fragment (and scale) requests alternate
       __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
 #pragma unroll
       for (int j = 0; j < T::TN; ++j) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+        if (LAST && j == 0) __builtin_amdgcn_sched_group_barrier(0x100, RPF + 2, 0);
+        else if (LAST) __builtin_amdgcn_sched_group_barrier(0x100, RPF + 1, 0);
+        else __builtin_amdgcn_sched_group_barrier(0x100, RPF, 0);
+      }
+      if constexpr (MXG && !LAST) {
+        // (same reason as above: keeps this slice's last row block in front of the next slice)
+        if constexpr (T::TN == 4) asm volatile("" : "+v"(acc[T::TM - 1][0]), "+v"(acc[T::TM - 1][1]), "+v"(acc[T::TM - 1][2]), "+v"(acc[T::TM - 1][3]));
+        else asm volatile("" : "+v"(acc[T::TM - 1][0]), "+v"(acc[T::TM - 1][1]));
+      }
+      if constexpr (LAST) {
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i) sca[i] = nsca[i];
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) scb[j] = nscb[j];
       }
     };
 
@@ -592,6 +670,12 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
           __builtin_amdgcn_s_waitcnt(0x0070);
         }
         __syncthreads();
+        if constexpr (MXG) {
+          if ((it + SC_LEAD) % T::SCG == 0) {
+            const int grp = (it + SC_LEAD) / T::SCG;
+            if (grp >= g0 + 2 && grp * T::SCG < it1) sc_dma(grp);   // (older than the operand copies below)
+          }
+        }
         if (it + S < it1 && !(p.debug & 1)) {
           OA::dma(sa, it + S, lds + stage * T::STAGE_BYTES, li.tid);
           OB::dma(sb, it + S, lds + stage * T::STAGE_BYTES + T::A_BYTES, li.tid);
@@ -602,182 +686,21 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         boundary();
       } else {
         if constexpr (T::KSUB == 1) {
-          block(std::integral_constant<int, 0>{}, sA, boundary, nA, nB, 0);
+          block(std::integral_constant<int, 0>{}, sA, boundary, nA, nB, 0, it + 1);
         } else if constexpr (T::KSUB == 2) {
-          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1);
-          block(std::integral_constant<int, 1>{}, sA, boundary, nA, nB, 0);
+          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1, it);
+          block(std::integral_constant<int, 1>{}, sA, boundary, nA, nB, 0, it + 1);
         } else {
           static_assert(T::KSUB == 4, "MFMA slices per K step");
-          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1);
-          block(std::integral_constant<int, 1>{}, sA, nothing, sA, sB, 2);
-          block(std::integral_constant<int, 2>{}, sA, nothing, sA, sB, 3);
-          block(std::integral_constant<int, 3>{}, sA, boundary, nA, nB, 0);
+          block(std::integral_constant<int, 0>{}, sA, nothing, sA, sB, 1, it);
+          block(std::integral_constant<int, 1>{}, sA, nothing, sA, sB, 2, it);
+          block(std::integral_constant<int, 2>{}, sA, nothing, sA, sB, 3, it);
+          block(std::integral_constant<int, 3>{}, sA, boundary, nA, nB, 0, it + 1);
         }
       }
       stage = nstage;
     };
     for (int it = it0; it < it1; ++it) kstep(it);
-  } else if constexpr (T::DMA) {
-    // fp4 with LDS-staged scales: copies run S-1 steps ahead, one barrier at the end of every K step
-    // (the scale registers leave no room for fragments that live across the barrier).
-    constexpr int S = T::STAGES;
-    constexpr int NG = OA::NCH + OB::NCH;
-    static_assert((S - 2) * NG <= 63, "vmcnt range");
-#pragma unroll
-    for (int s = 0; s < S - 1; ++s) {
-      if (it0 + s < it1) {
-        OA::dma(sa, it0 + s, lds + s * T::STAGE_BYTES, li.tid);
-        OB::dma(sb, it0 + s, lds + s * T::STAGE_BYTES + T::A_BYTES, li.tid);
-      }
-    }
-    // ---- MX scales through LDS (fp4).  One scale group = 32 scale bytes of every tile row = the
-    // scales of SCG consecutive K steps.  A group is copied raw ([step][lane group][KSUB bytes] per
-    // row), transposed in place to [lane group][step][KSUB bytes] (8 contiguous bytes per lane group)
-    // and then read with one 8-byte LDS load per lane and row block.
-    uint8_t* sc_lds = lds + T::LDS_BYTES;
-    constexpr int NQ = (T::BM + T::BN) * (T::SC_GB / 16);          // 16-byte scale chunks per group
-    constexpr int NSCH = MXG ? (NQ + T::THREADS - 1) / T::THREADS : 1;
-    constexpr int NTR = MXG ? ((T::BM + T::BN) * 4 + T::THREADS - 1) / T::THREADS : 1;   // (row, lane group) items
-    const uint8_t* scp[NSCH];
-    int reg_group = -1, lds_group = -1, read_it = -1, dma_it = -1;
-    bool lds_ready = false;
-    if constexpr (MXG) {
-#pragma unroll
-      for (int i = 0; i < NSCH; ++i) {
-        const int q = i * T::THREADS + li.tid;
-        const int row = q / (T::SC_GB / 16), part = q % (T::SC_GB / 16);
-        if (row < T::BM) scp[i] = p.mxa + (int64_t)min(tc.m0 + row, tc.m_lim - 1) * p.mxa_sr + part * 16;
-        else scp[i] = p.mxb + (int64_t)min(tc.n0 + row - T::BM, tc.n_lim - 1) * p.mxb_sr + part * 16;
-      }
-    }
-    auto sc_dma = [&](int grp) {
-      if constexpr (MXG) {
-        const int wave_slot = __builtin_amdgcn_readfirstlane(li.tid & ~63);
-        const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)sc_lds);
-#pragma unroll
-        for (int i = 0; i < NSCH; ++i) {
-          if (NQ % T::THREADS != 0 && i * T::THREADS + wave_slot >= NQ) continue;
-          const uint32_t dst = lds0 + (uint32_t)((i * T::THREADS + wave_slot) * 16);
-          const uint8_t* src = scp[i] + (int64_t)grp * T::SC_GB;
-          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory", "m0");
-        }
-      }
-    };
-    // in place: the four lanes that own one row are neighbours in a wave, and a wave's reads of an
-    // item all complete before its writes of that item are issued (the writes consume the reads)
-    auto sc_transpose = [&]() {
-      if constexpr (MXG) {
-        uint32_t w0[NTR], w1[NTR];
-#pragma unroll
-        for (int i = 0; i < NTR; ++i) {
-          const int idx = i * T::THREADS + li.tid;
-          w0[i] = w1[i] = 0;
-          if (((T::BM + T::BN) * 4) % T::THREADS != 0 && idx >= (T::BM + T::BN) * 4) continue;
-          const uint8_t* b = sc_lds + (idx >> 2) * T::SC_GB + (idx & 3) * T::KSUB;
-#pragma unroll
-          for (int s = 0; s < T::SCG; ++s) {
-            uint32_t v = (T::KSUB == 2) ? (uint32_t)(*(const uint16_t*)(b + s * T::CPR)) : (uint32_t)(*(b + s * T::CPR));
-            if ((s * T::KSUB) >> 2) w1[i] |= v << (8 * ((s * T::KSUB) & 3));
-            else w0[i] |= v << (8 * ((s * T::KSUB) & 3));
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < NTR; ++i) {
-          const int idx = i * T::THREADS + li.tid;
-          if (((T::BM + T::BN) * 4) % T::THREADS != 0 && idx >= (T::BM + T::BN) * 4) continue;
-          *(uint2*)(sc_lds + (idx >> 2) * T::SC_GB + (idx & 3) * 8) = uint2{w0[i], w1[i]};
-        }
-      }
-    };
-    auto sc_read = [&]() {
-      if constexpr (MXG) {
-#pragma unroll
-        for (int i = 0; i < T::TM; ++i) {
-          uint2 v = *(const uint2*)(sc_lds + (li.wm0 + i * 16 + li.r) * T::SC_GB + li.g * 8);
-          ga[i][0] = v.x; ga[i][1] = v.y;
-        }
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) {
-          uint2 v = *(const uint2*)(sc_lds + (T::BM + li.wn0 + j * 16 + li.r) * T::SC_GB + li.g * 8);
-          gb[j][0] = v.x; gb[j][1] = v.y;
-        }
-      }
-    };
-    static_assert(!MXG || T::KSUB <= 2, "LDS-staged scales hold 8 bytes per lane and row block");
-
-    sc_dma(it0 / T::SCG);
-    lds_group = it0 / T::SCG;
-    wait_vm0();
-    __syncthreads();
-    sc_transpose();
-    lds_ready = true;
-    __syncthreads();
-    int stage = 0;
-    // one K step; SC is the step's compile-time position in its scale group, or -1 (found at run time)
-    auto kstep = [&](int it, auto SC) {
-      constexpr int SCV = decltype(SC)::value;
-      const int nxt = it + S - 1;
-      int wstage = stage + S - 1; if (wstage >= S) wstage -= S;
-      const int grp = it / T::SCG;
-      if (grp != reg_group) {
-        if (lds_group != grp) {  // only right after a segment start: nobody could prefetch this group
-          sc_dma(grp);
-          wait_vm0();
-          __syncthreads();
-          lds_group = grp;
-          lds_ready = false;
-        }
-        if (!lds_ready) {
-          sc_transpose();
-          lds_ready = true;
-          __syncthreads();
-        }
-        sc_read();
-        reg_group = grp;
-        read_it = it;
-      } else if (lds_group == grp && it > read_it && (grp + 1) * T::SCG < it1) {
-        sc_dma(grp + 1);       // every wave has consumed group grp (a barrier has passed since)
-        lds_group = grp + 1;
-        lds_ready = false;
-        dma_it = it;
-      } else if (lds_group == grp + 1 && !lds_ready && it > dma_it) {
-        sc_transpose();        // the copy landed with the wait that closed step dma_it
-        lds_ready = true;
-      }
-      if constexpr (SCV < 0) {
-        const int sidx = (it % T::SCG) * T::KSUB;
-        const int sh = 8 * (sidx & 3);
-#pragma unroll
-        for (int i = 0; i < T::TM; ++i) sca[i] = ((sidx >> 2) ? ga[i][1] : ga[i][0]) >> sh;
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j) scb[j] = ((sidx >> 2) ? gb[j][1] : gb[j][0]) >> sh;
-      }
-      if (nxt < it1 && !(p.debug & 1)) {
-        OA::dma(sa, nxt, lds + wstage * T::STAGE_BYTES, li.tid);
-        OB::dma(sb, nxt, lds + wstage * T::STAGE_BYTES + T::A_BYTES, li.tid);
-      }
-      if (!(p.debug & 2)) compute(SC, lds + stage * T::STAGE_BYTES, lds + stage * T::STAGE_BYTES + T::A_BYTES);
-      wait_vm0();   // (the scale copy is the youngest load of a step: nothing may stay in flight)
-      __syncthreads();
-      stage = (stage + 1 == S) ? 0 : stage + 1;
-    };
-    if constexpr (WHOLE) {
-      // whole tiles of the fast fp4 kernels: k_iters is a multiple of the scale group (K % 1024 == 0)
-      for (int it = it0; it < it1; it += T::SCG) {
-        kstep(it, std::integral_constant<int, 0>{});
-        kstep(it + 1, std::integral_constant<int, 1>{});
-        kstep(it + 2, std::integral_constant<int, 2>{});
-        kstep(it + 3, std::integral_constant<int, 3>{});
-        if constexpr (T::SCG == 8) {
-          kstep(it + 4, std::integral_constant<int, 4>{});
-          kstep(it + 5, std::integral_constant<int, 5>{});
-          kstep(it + 6, std::integral_constant<int, 6>{});
-          kstep(it + 7, std::integral_constant<int, 7>{});
-        }
-      }
-    } else {
-      for (int it = it0; it < it1; ++it) kstep(it, std::integral_constant<int, -1>{});
-    }
   } else {
     v4i ra[OA::NREG], rb[OB::NREG];
     uint8_t* sA0 = lds;
@@ -796,7 +719,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::gload(rb, sb, it + 1, p.KU, li.tid);
         load_scales(it + 1, nsca, nscb);
       }
-      if (!(p.debug & 2)) compute(std::integral_constant<int, -1>{}, sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
+      if (!(p.debug & 2)) compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
       if (has_next) {
         OA::sstore(sA0 + (cur ^ 1) * T::STAGE_BYTES, ra, li.tid);
         OB::sstore(sB0 + (cur ^ 1) * T::STAGE_BYTES, rb, li.tid);

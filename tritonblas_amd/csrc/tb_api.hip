@@ -197,8 +197,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   const Variant* v = nullptr;
   bool fast = alay >= 0 && blay >= 0 && (KU % (bk / epu) == 0);
   if (j.dt == TB_FP4_E2M1) {
-    // the fast fp4 kernels stage 32 scale bytes per row at a time through LDS with 16-byte copies
-    const bool mx_ok = j.mxa_sk == 1 && j.mxb_sk == 1 && (j.K / 32) % 32 == 0 && j.mxa_sr % 16 == 0 && j.mxb_sr % 16 == 0 &&
+    // the fast fp4 kernels stage 16 scale bytes per row at a time through LDS with 16-byte copies
+    const bool mx_ok = j.mxa_sk == 1 && j.mxb_sk == 1 && (j.K / 32) % 16 == 0 && j.mxa_sr % 16 == 0 && j.mxb_sr % 16 == 0 &&
                        ((uintptr_t)j.mxa % 16) == 0 && ((uintptr_t)j.mxb % 16) == 0;
     const char* e = getenv("TB_NO_MXLDS");
     if (!mx_ok || (e && atoi(e))) fast = false;
