@@ -51,6 +51,18 @@ enum {
   TB_SCHED_STREAMK = 2        /* data parallel tiles + Stream-K tail     (matmul.py:202-366)        */
 };
 
+/* How work-stealing workgroups find tiles (kernels/persistent_gemm_work_stealing.py). */
+enum tb_ws_mode {
+  TB_WS_QUEUES = 0,        /* one queue per XCD x slot (:296-318); a workgroup whose queues ran dry
+                              goes on to the other queues (this library's addition)                  */
+  TB_WS_GLOBAL_ATOMIC = 1, /* GLOBAL_ATOMIC: one counter, entry i is tile chiplet_transform(i) (:292-295, :321) */
+  TB_WS_HIERARCHICAL = 2   /* HIERARCHICAL: a queue of ws_local_tiles_per_xcd tiles per XCD, then one
+                              shared pool of ws_global_tiles (:106-291; split: origami.py:288-311);
+                              a workgroup that finds both empty looks into the other XCDs' queues, so
+                              every tile is computed whatever the mask switches off (this library's
+                              addition)                                                              */
+};
+
 /* ---- hardware descriptor (replaces origami.get_hardware_for_device, origami.py:166) --------- */
 typedef struct tb_hw {
   int32_t n_cu;          /* compute units                                   */
@@ -121,6 +133,14 @@ typedef struct tb_gemm_desc {
   size_t workspace_bytes;
   uint32_t epoch;             /* Stream-K: must differ from the previous launch on this workspace    */
   uint32_t spin_limit;        /* Stream-K: bound on flag polls per wait; 0 = default                 */
+  /* work stealing only (config.py:23, persistent_gemm_work_stealing.py:70-81): */
+  const int32_t* cu_mask;     /* device int32[cu_mask_len] or NULL; workgroup i leaves at once when
+                                 cu_mask[i] == 0.  With grid == 0 the launch has cu_mask_len workgroups
+                                 (the reference launches one per CU and masks by program id)          */
+  int32_t cu_mask_len;
+  int32_t ws_mode;            /* TB_WS_*                                                            */
+  int32_t ws_local_tiles_per_xcd, ws_global_tiles;  /* TB_WS_HIERARCHICAL: num_xcds * local + global
+                                 must equal the tile count                                           */
 } tb_gemm_desc;
 
 /* C = cast((A @ B) * a_scale[:,None] * b_scale[None,:] + bias[None,:]), fp32 accumulate.
@@ -195,6 +215,13 @@ int tb_hadamard_mxfp4_quant(const tb_quant_desc* desc, void* stream);
  * tb_default_panel gives the panel width tb_gemm uses for a launch grid. */
 int tb_tile_coords(int32_t tile, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t panel_n, int32_t* pm, int32_t* pn);
 int tb_default_panel(int32_t grid, int32_t chunk, int32_t group_m);
+
+/* Host-side evaluation of the work-stealing queues: queue `queue` of a launch over total_tiles tiles
+ * (TB_WS_QUEUES: queue = xcd * counters_per_xcd + slot; TB_WS_GLOBAL_ATOMIC: queue 0;
+ * TB_WS_HIERARCHICAL: queue = xcd, or num_xcds for the shared pool).  *count = entries of the queue,
+ * *tile = tile id of entry idx (or -1 when idx >= *count). */
+int tb_ws_queue_tile(int32_t ws_mode, int32_t queue, int32_t idx, int32_t total_tiles, int32_t num_xcds,
+                     int32_t counters_per_xcd, int32_t local_tiles_per_xcd, int32_t* count, int32_t* tile);
 
 /* ---- misc ----------------------------------------------------------------------------------- */
 const char* tb_status_string(int status);

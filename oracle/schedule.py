@@ -107,3 +107,39 @@ def grouped_tile_lookup(tile_id, offsets, block_m, tiles_n):
             return e, local % mb, local // mb
         acc += cnt
     return None
+
+
+def ws_global_atomic_tile(raw_idx, total_tiles, num_xcds):
+    """Tile a work-stealing workgroup gets for counter value raw_idx in GLOBAL_ATOMIC mode
+    (reference kernels/persistent_gemm_work_stealing.py:292-295, 321)."""
+    return chiplet_transform(raw_idx, total_tiles, num_xcds)
+
+
+def ws_hierarchical_tile(xcd, raw_idx, level, local_tiles_per_xcd, num_xcds):
+    """HIERARCHICAL mode (reference persistent_gemm_work_stealing.py:106-122, 211-216): level 1 takes
+    from the XCD's own run of local_tiles_per_xcd tiles, level 2 from the pool behind all local runs."""
+    if level == 1:
+        return xcd * local_tiles_per_xcd + raw_idx
+    return local_tiles_per_xcd * num_xcds + raw_idx
+
+
+def hierarchical_split(total_tiles, hw_cus, num_xcds):
+    """(local_per_xcd, global_tiles), reference origami.py:288-311 verbatim in arithmetic."""
+    tiles_per_cu = total_tiles / max(hw_cus, 1)
+    local_frac = max(0.5, 1.0 - max(0.0, tiles_per_cu - 4.0) * 0.05)
+    local_per_xcd = int(total_tiles * local_frac) // num_xcds
+    local_per_xcd = max(local_per_xcd, 1)
+    return local_per_xcd, total_tiles - local_per_xcd * num_xcds
+
+
+def build_balanced_hex_mask(remove_per_xcd, num_xcds, cus_per_xcd):
+    """CU-mask string that removes remove_per_xcd CUs from every XCD (CU bit i belongs to XCD
+    i % num_xcds; reference benchmarks/common.py:34-45)."""
+    if remove_per_xcd == 0:
+        return ""
+    total = num_xcds * cus_per_xcd
+    mask = (1 << total) - 1
+    for i in range(remove_per_xcd):
+        for xcd in range(num_xcds):
+            mask &= ~(1 << (num_xcds * i + xcd))
+    return f"0x{mask:x}"

@@ -57,3 +57,32 @@ def test_driver_runs_a_shape_list_with_correctness_check(tmp_path, flags):
     assert len(rows) == len(cases) and list(rows[0].keys()) == REFERENCE_COLUMNS
     want_mode = "work_stealing" if "--work-stealing" in flags else ("streamk" if "--enable-streamk" in flags else "persistent")
     assert all(r["mode"] == want_mode and float(r["tritonblas_gflops"]) > 0 for r in rows)
+
+
+def test_cu_sweep_steps():
+    from tritonblas_amd.benchmarks.matmul_bench import cu_sweep_steps, _fieldnames
+    assert cu_sweep_steps(256, 8, 32, 3) == [256, 248, 240, 232]
+    assert cu_sweep_steps(304, 8, 38, 34) == [304 - 8 * r for r in range(35)]          # the reference's MI300X default
+    assert cu_sweep_steps(256, 8, 32, 100)[-1] == 8                                    # at least one CU per XCD stays
+    assert _fieldnames([{"active_cus": 8, "m": 1}]) == ["active_cus"] + REFERENCE_COLUMNS
+    assert _fieldnames([{"m": 1}]) == REFERENCE_COLUMNS and _fieldnames([]) == REFERENCE_COLUMNS
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("flags", [["--work-stealing"], ["--work-stealing", "--global-atomic"], ["--work-stealing", "--hierarchical"], []])
+def test_driver_cu_sweep(tmp_path, flags):
+    from tritonblas_amd.benchmarks import matmul_bench
+    from tritonblas_amd.benchmarks.common import get_cu_info
+    print(f"bench driver cu sweep {flags}", flush=True)
+    cases = [
+        {"m": 1024, "n": 1024, "k": 512, "in_dtype": "bfloat16", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+        {"m": 512, "n": 768, "k": 1024, "in_dtype": "float8_e4m3fn", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+    ]
+    src, dst = tmp_path / "shapes.yaml", tmp_path / "out.csv"
+    src.write_text(yaml.safe_dump(cases))
+    matmul_bench.main(["--input-yaml", str(src), "--output-csv", str(dst), "--checkcorrectness", "--n-warmup", "1",
+                       "--n-repeat", "2", "--cu-sweep", "--cu-sweep-max-remove", "2"] + flags)
+    rows = list(csv.DictReader(dst.open()))
+    full, xcds, _ = get_cu_info(0)
+    assert list(rows[0].keys()) == ["active_cus"] + REFERENCE_COLUMNS
+    assert [int(r["active_cus"]) for r in rows] == [full] * 2 + [full - xcds] * 2 + [full - 2 * xcds] * 2

@@ -185,6 +185,96 @@ def test_work_stealing_is_bit_identical_to_static(m, n, k, dtype):
         assert torch.equal(c0, c1), f"launch {rep}"
 
 
+@pytest.mark.parametrize("mode", ["global_atomic", "hierarchical"])
+@pytest.mark.parametrize("m,n,k", [(768, 1024, 512), (2048, 2048, 256), (300, 200, 192), (16, 16, 4096), (4096, 4096, 128)])
+def test_work_stealing_queue_modes_are_bit_identical_to_static(mode, m, n, k):
+    """One shared counter, and XCD-local queues followed by a shared pool: every tile is computed exactly
+    once whichever workgroup gets it, so C equals the static schedule's bit for bit; the counters
+    (the pool's included) rearm themselves."""
+    import tritonblas_amd as tb
+    _say(f"work stealing {mode} {m}x{n}x{k}")
+    dtype = torch.bfloat16
+    a, b = _rand((m, k), dtype, 11, 0.5).cuda(), _rand((k, n), dtype, 12, 0.5).cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device)
+    cfg = tb.matmul_preamble(sel)
+    setattr(cfg, mode, True)
+    c0 = torch.zeros(m, n, dtype=dtype, device="cuda")
+    tb.matmul_lt(a, b, c0, sel)
+    for rep in range(3):
+        c1 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        tb.matmul_lt(a, b, c1, sel, cfg, work_stealing=True)
+        assert torch.equal(c0, c1), f"launch {rep}"
+    # the same workspace serves the other modes afterwards
+    cfg.global_atomic = cfg.hierarchical = False
+    c2 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+    tb.matmul_lt(a, b, c2, sel, cfg, work_stealing=True)
+    assert torch.equal(c0, c2)
+
+
+@pytest.mark.parametrize("mode", ["queues", "global_atomic", "hierarchical"])
+@pytest.mark.parametrize("active", [1, 7, 64, 200])
+def test_work_stealing_with_masked_workgroups(mode, active):
+    """active_cus < total_cus: the masked-out workgroups leave at once and the others take every tile
+    (also the tiles of queues whose own workgroups are all masked out)."""
+    import tritonblas_amd as tb
+    m, n, k = 1024, 1536, 256
+    _say(f"work stealing mask active={active} {mode}")
+    dtype = torch.float16
+    a, b = _rand((m, k), dtype, 21, 0.5).cuda(), _rand((k, n), dtype, 22, 0.5).cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device, active_cus=active)
+    cfg = tb.matmul_preamble(sel)
+    assert cfg.mask.numel() == sel._N_CU and int(cfg.mask.sum()) == active and cfg.active_mask() is cfg.mask
+    if mode != "queues":
+        setattr(cfg, mode, True)
+    c0 = torch.zeros(m, n, dtype=dtype, device="cuda")
+    tb.matmul_lt(a, b, c0, sel)
+    for rep in range(2):
+        c1 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+        tb.matmul_lt(a, b, c1, sel, cfg, work_stealing=True)
+        assert torch.equal(c0, c1), f"launch {rep}"
+    # a caller-made mask with holes
+    holes = torch.zeros(sel._N_CU, dtype=torch.int32)
+    holes[3::5] = 1
+    cfg.mask = holes.cuda()
+    c2 = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+    tb.matmul_lt(a, b, c2, sel, cfg, work_stealing=True)
+    assert torch.equal(c0, c2)
+
+
+def test_work_stealing_bad_mask_and_split_are_refused():
+    import ctypes as C
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    m = n = k = 512
+    a, b = _rand((m, k), torch.float16, 1).cuda(), _rand((k, n), torch.float16, 2).cuda()
+    c = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, a.dtype, a.dtype, a.device)
+    cfg = tb.matmul_preamble(sel)
+    cfg.mask = torch.ones(8, dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError, match="int32"):
+        tb.matmul_lt(a, b, c, sel, cfg, work_stealing=True)
+    # through the C ABI: a grid larger than the mask, and a split that does not add up
+    d = _lib.tb_gemm_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+    d.a_type = d.b_type = d.c_type = _lib.tb_dtype(torch.float16)
+    d.m, d.n, d.k = m, n, k
+    d.a_stride_m, d.a_stride_k, d.b_stride_k, d.b_stride_n, d.c_stride_m, d.c_stride_n = k, 1, n, 1, n, 1
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.schedule = _lib.TB_SCHED_WORK_STEALING
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+    mask = torch.ones(16, dtype=torch.int32, device="cuda")
+    d.cu_mask, d.cu_mask_len, d.grid = mask.data_ptr(), 16, 32
+    lib = _lib.load()
+    assert lib.tb_gemm(d, None) == -10          # TB_ERR_BAD_ARGUMENT
+    d.grid = 0
+    d.ws_mode, d.ws_local_tiles_per_xcd, d.ws_global_tiles = _lib.TB_WS_HIERARCHICAL, 1, 1
+    assert lib.tb_gemm(d, None) == -7           # TB_ERR_BAD_SCHEDULE
+    d.ws_mode = 5
+    assert lib.tb_gemm(d, None) == -7
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("m,n,k,grid", [(256, 256, 4096, 64), (128, 128, 8192, 256), (768, 1024, 512, 100), (300, 200, 1920, 37),
                                        (32, 512, 8192, 256), (64, 64, 64, 8)])
 @pytest.mark.parametrize("dtype", DTYPES)

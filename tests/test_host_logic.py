@@ -229,3 +229,125 @@ def test_custom_op_fake_implementations_propagate_shapes():
         assert tb.matmul(a, b, out=out) is None and tb.addmm(bias, a, b, out=out) is None
         with pytest.raises(Exception, match="Incompatible A-B Dimensions"):
             tb.matmul(a, torch.empty(31, 48, device="cuda", dtype=torch.bfloat16))
+
+
+# ---- work-stealing queues (host evaluation through the C ABI) ------------------------------------
+from oracle import schedule as OS
+
+TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
+
+
+def _queue(lib, mode, q, total, X, S, local):
+    cnt, tile = C.c_int32(-1), C.c_int32(-1)
+    assert lib.tb_ws_queue_tile(mode, q, 0, total, X, S, local, C.byref(cnt), C.byref(tile)) == 0
+    out = []
+    for i in range(cnt.value):
+        c2 = C.c_int32(-1)
+        assert lib.tb_ws_queue_tile(mode, q, i, total, X, S, local, C.byref(c2), C.byref(tile)) == 0
+        assert c2.value == cnt.value
+        out.append(tile.value)
+    assert lib.tb_ws_queue_tile(mode, q, cnt.value, total, X, S, local, C.byref(c2 if cnt.value else cnt), C.byref(tile)) == 0
+    assert tile.value == -1
+    return out
+
+
+@pytest.mark.parametrize("total,X,S", [(1, 8, 4), (7, 8, 1), (64, 8, 8), (1000, 8, 4), (3584, 8, 1), (333, 4, 2), (50, 1, 3)])
+def test_ws_flat_queues_follow_the_reference_ranges_and_cover_every_tile_once(total, X, S):
+    lib = _load()
+    seen = []
+    for pid in range(X * S):   # workgroups 0..X*S-1 sit on distinct queues
+        q, first, bound = OS.ws_slot_range(pid, total, X, S)
+        got = _queue(lib, TB_WS_QUEUES, q, total, X, S, 0)
+        assert got == list(range(first, first + bound))
+        seen += got
+    assert sorted(seen) == list(range(total))
+
+
+@pytest.mark.parametrize("total,X", [(1, 8), (7, 8), (64, 8), (1001, 8), (333, 4), (50, 1)])
+def test_ws_global_atomic_queue_is_the_chiplet_transform_of_the_counter(total, X):
+    lib = _load()
+    got = _queue(lib, TB_WS_GLOBAL_ATOMIC, 0, total, X, 4, 0)
+    assert got == [OS.ws_global_atomic_tile(i, total, X) for i in range(total)]
+    assert sorted(got) == list(range(total))
+    # workgroup ids dealt round-robin to XCDs: consecutive counter values alternate between XCD runs
+    if X > 1 and total >= 2 * X and total % X == 0:
+        assert got[1] - got[0] == total // X
+
+
+@pytest.mark.parametrize("total,X,local", [(1024, 8, 128), (1024, 8, 100), (9, 8, 1), (5, 8, 0), (3584, 8, 224), (77, 4, 10)])
+def test_ws_hierarchical_queues(total, X, local):
+    lib = _load()
+    seen = []
+    for xcd in range(X):
+        got = _queue(lib, TB_WS_HIERARCHICAL, xcd, total, X, 4, local)
+        assert got == [OS.ws_hierarchical_tile(xcd, i, 1, local, X) for i in range(local)]
+        seen += got
+    pool = _queue(lib, TB_WS_HIERARCHICAL, X, total, X, 4, local)
+    assert pool == [OS.ws_hierarchical_tile(0, i, 2, local, X) for i in range(total - X * local)]
+    assert sorted(seen + pool) == list(range(total))
+
+
+def test_ws_queue_tile_rejects_bad_arguments():
+    lib = _load()
+    cnt, tile = C.c_int32(), C.c_int32()
+    TB_ERR_NULL_POINTER, TB_ERR_BAD_ARGUMENT = -1, -10
+    assert lib.tb_ws_queue_tile(3, 0, 0, 10, 8, 4, 0, C.byref(cnt), C.byref(tile)) == TB_ERR_BAD_ARGUMENT
+    assert lib.tb_ws_queue_tile(0, 32, 0, 10, 8, 4, 0, C.byref(cnt), C.byref(tile)) == TB_ERR_BAD_ARGUMENT
+    assert lib.tb_ws_queue_tile(1, 1, 0, 10, 8, 4, 0, C.byref(cnt), C.byref(tile)) == TB_ERR_BAD_ARGUMENT
+    assert lib.tb_ws_queue_tile(2, 0, 0, 10, 8, 4, 2, C.byref(cnt), C.byref(tile)) == TB_ERR_BAD_ARGUMENT   # 8*2 > 10
+    assert lib.tb_ws_queue_tile(0, 0, 0, 10, 8, 4, 0, None, C.byref(tile)) == TB_ERR_NULL_POINTER
+
+
+def test_hierarchical_split_known_answers():
+    # <= 4 tiles per CU: everything local; 14 tiles per CU and beyond: half
+    assert OS.hierarchical_split(1024, 256, 8) == (128, 0)
+    assert OS.hierarchical_split(512, 256, 8) == (64, 0)
+    assert OS.hierarchical_split(3584, 256, 8) == (224, 1792)          # 14 per CU -> frac 0.5
+    assert OS.hierarchical_split(256 * 20, 256, 8) == (320, 2560)      # floor at one half
+    lp, g = OS.hierarchical_split(2048, 256, 8)                        # 8 per CU -> frac 0.8
+    assert (lp, g) == (int(2048 * 0.8) // 8, 2048 - 8 * (int(2048 * 0.8) // 8))
+
+
+@pytest.mark.parametrize("m,n,k", [(8192, 8192, 8192), (8192, 28672, 8192), (4096, 4096, 4096), (256, 256, 256), (16384, 16384, 1024)])
+def test_selector_hierarchical_split_matches_the_reference_formula(m, n, k):
+    import tritonblas_amd as tb
+    sel = tb.OrigamiMatmulSelector(m, n, k, torch.bfloat16, torch.bfloat16, torch.bfloat16, "cpu")
+    total = -(-m // sel.block_m) * -(-n // sel.block_n)
+    hw = sel._hardware._c.num_xcd * sel._hardware._c.cu_per_xcd
+    X = sel.num_sms
+    want = OS.hierarchical_split(total, hw, X)
+    got = sel.hierarchical_split(X)
+    assert got[0] * X + got[1] == total and got[0] >= 0 and got[1] >= 0
+    if want[1] >= 0:
+        assert got == want
+    else:   # fewer tiles than XCDs: the reference formula overshoots, the selector keeps the split valid
+        assert got == (total // X, total - X * (total // X))
+
+
+@pytest.mark.parametrize("remove,X,per", [(0, 8, 32), (1, 8, 32), (5, 8, 32), (31, 8, 32), (3, 4, 20), (2, 1, 7)])
+def test_balanced_cu_mask(remove, X, per):
+    from tritonblas_amd.benchmarks.common import build_balanced_hex_mask
+    s = build_balanced_hex_mask(remove, X, per)
+    assert s == OS.build_balanced_hex_mask(remove, X, per)
+    if remove == 0:
+        assert s == ""
+        return
+    v = int(s, 16)
+    assert v < (1 << (X * per))
+    for xcd in range(X):   # CU bit i sits on XCD i % X: every XCD loses exactly `remove` CUs, the lowest ones
+        bits = [(v >> i) & 1 for i in range(xcd, X * per, X)]
+        assert bits == [0] * remove + [1] * (per - remove)
+
+
+def test_matmul_config_mask_rules():
+    import tritonblas_amd as tb
+    from tritonblas_amd.config import MatmulConfig
+    cfg = MatmulConfig(device=torch.device("cpu"), workspace=None)
+    assert cfg.mask is None and cfg.active_mask() is None and not cfg.global_atomic and not cfg.hierarchical
+    m = torch.ones(8, dtype=torch.int32)
+    cfg.mask = m            # a mask the caller assigns is used
+    assert cfg.active_mask() is m
+    cfg.mask = None
+    assert cfg.active_mask() is None
+    cfg2 = MatmulConfig(device=torch.device("cpu"), workspace=None, mask=m, use_mask=False)   # what matmul_preamble does with all CUs active
+    assert cfg2.mask is m and cfg2.active_mask() is None

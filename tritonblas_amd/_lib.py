@@ -18,11 +18,12 @@ TB_ERR_NULL_POINTER, TB_ERR_BAD_SHAPE, TB_ERR_BAD_DTYPE, TB_ERR_BAD_LAYOUT, TB_E
 TB_ERR_WORKSPACE, TB_ERR_BAD_SCHEDULE, TB_ERR_LAUNCH, TB_ERR_NO_DEVICE, TB_ERR_BAD_ARGUMENT = -6, -7, -8, -9, -10
 TB_F16, TB_BF16, TB_FP8_E4M3, TB_FP4_E2M1, TB_F32 = 0, 1, 2, 3, 4
 TB_SCHED_PERSISTENT, TB_SCHED_WORK_STEALING, TB_SCHED_STREAMK = 0, 1, 2
+TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
 
 EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
-    "tb_tile_coords", "tb_default_panel",
+    "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile",
 ]
 
 
@@ -55,7 +56,9 @@ class tb_gemm_desc(C.Structure):
                 ("block_m", C.c_int32), ("block_n", C.c_int32), ("block_k", C.c_int32), ("group_m", C.c_int32),
                 ("num_xcds", C.c_int32), ("schedule", C.c_int32), ("grid", C.c_int32),
                 ("counters_per_xcd", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-                ("epoch", C.c_uint32), ("spin_limit", C.c_uint32)]
+                ("epoch", C.c_uint32), ("spin_limit", C.c_uint32), ("cu_mask", C.c_void_p),
+                ("cu_mask_len", C.c_int32), ("ws_mode", C.c_int32), ("ws_local_tiles_per_xcd", C.c_int32),
+                ("ws_global_tiles", C.c_int32)]
 
 
 class tb_gemm_fp4_desc(C.Structure):
@@ -112,6 +115,7 @@ def load():
     lib.tb_hadamard_mxfp4_quant.argtypes = [C.POINTER(tb_quant_desc), C.c_void_p]
     lib.tb_tile_coords.argtypes = [C.c_int32] * 5 + [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.tb_default_panel.argtypes = [C.c_int32] * 3
+    lib.tb_ws_queue_tile.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32)] * 2
     if lib.tb_abi_version() != 1:
         raise RuntimeError("libtritonblas_amd.so ABI version mismatch")
     _lib = lib

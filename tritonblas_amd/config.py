@@ -17,14 +17,36 @@ _CTL_BYTES = 256
 
 
 class MatmulConfig:
+    """``mask``: int32 per-workgroup enable mask of the work-stealing launch (1 = takes tiles, 0 = leaves
+    at once; reference config.py:23).  A mask that ``matmul_preamble`` made for a selector with all CUs
+    active is not handed to the kernel (the launch then keeps its default, occupancy-filling grid);
+    a mask with masked-out entries, or one the caller assigns, is, and the launch has one workgroup
+    per mask entry like the reference's.  ``global_atomic`` / ``hierarchical`` pick the single-counter
+    and the XCD-local-then-shared-pool queueing of the reference's work-stealing kernel."""
+
     def __init__(self, device: torch.device, workspace: torch.Tensor, selector=None, mask: torch.Tensor = None,
-                 global_atomic: bool = False):
+                 global_atomic: bool = False, hierarchical: bool = False, use_mask: bool = None):
         self.device = device
         self.workspace = workspace
         self.selector = selector
-        self.mask = mask
+        self._mask = mask
+        self._use_mask = (mask is not None) if use_mask is None else use_mask
         self.global_atomic = global_atomic
+        self.hierarchical = hierarchical
         self.epoch = 0
+
+    @property
+    def mask(self):
+        return self._mask
+
+    @mask.setter
+    def mask(self, value):
+        self._mask = value
+        self._use_mask = value is not None
+
+    def active_mask(self):
+        """The mask the kernel should look at, or None."""
+        return self._mask if self._use_mask else None
 
     def ensure(self, nbytes: int):
         """Grow the workspace to at least nbytes (zero-initialised)."""
@@ -100,4 +122,4 @@ def matmul_preamble(selector, device: torch.device = None) -> MatmulConfig:
     mask = torch.ones(n_cu, dtype=torch.int32, device=device)
     if active < n_cu:
         mask[active:] = 0
-    return MatmulConfig(device=device, workspace=workspace, selector=selector, mask=mask)
+    return MatmulConfig(device=device, workspace=workspace, selector=selector, mask=mask, use_mask=active < n_cu)

@@ -20,6 +20,7 @@ typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
 enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4 };
 enum : int { MODE_STATIC = 0, MODE_WS = 1, MODE_SK = 2, MODE_GROUPED = 3 };
+enum : int { WS_QUEUES = 0, WS_GLOBAL = 1, WS_HIERARCHICAL = 2 };   // how work-stealing workgroups find tiles
 enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
 
 // Word offsets inside the control block at the head of a workspace.
@@ -62,6 +63,8 @@ struct GemmParams {
   int32_t* counters;
   int32_t counters_per_xcd;
   const int32_t* cu_mask;
+  int32_t ws_mode;               // WS_*
+  int32_t ws_local, ws_global;   // hierarchical: tiles per XCD-local queue, tiles in the shared pool behind them
   // grouped
   const int32_t* group_offsets;
   int32_t num_groups;
@@ -139,6 +142,40 @@ __device__ __forceinline__ int chiplet_transform_chunked(int pid, int num_wg, in
   int local = pid / num_xcds;
   int chunk_idx = local / chunk, pos = local % chunk, xcd = pid % num_xcds;
   return chunk_idx * block + xcd * chunk + pos;
+}
+
+// pid -> position when workgroup ids are dealt round-robin to the XCDs: ids of one XCD become contiguous
+__host__ __device__ __forceinline__ int chiplet_transform(int pid, int num_wg, int num_xcds) {
+  int xcd = pid % num_xcds, pos = pid / num_xcds;
+  int min_per = num_wg / num_xcds, extra = num_wg % num_xcds;
+  return xcd * min_per + (xcd < extra ? xcd : extra) + pos;
+}
+
+// Work-stealing queues.  WS_QUEUES: queue (xcd, slot) owns a contiguous run of the tile list: the list
+// is cut into num_xcds parts and every part into S slots.  WS_GLOBAL: one queue over all tiles, entry
+// idx is tile chiplet_transform(idx).  WS_HIERARCHICAL: queue xcd owns tiles [xcd*local, (xcd+1)*local),
+// queue num_xcds (the shared pool) the rest.  Returns the queue's first tile and length.
+__host__ __device__ __forceinline__ void ws_queue_range(int mode, int queue, int total, int X, int S, int local, int& first, int& count) {
+  if (mode == WS_GLOBAL) { first = 0; count = queue == 0 ? total : 0; return; }
+  if (mode == WS_HIERARCHICAL) {
+    if (queue < X) { first = queue * local; count = local; }
+    else { first = X * local; count = queue == X ? total - X * local : 0; }
+    if (count < 0) count = 0;
+    return;
+  }
+  const int qx = queue / S, qs = queue % S;
+  const int per_xcd = (total + X - 1) / X;
+  const int xbase = qx * per_xcd;
+  int xcnt = (xbase + per_xcd < total ? xbase + per_xcd : total) - xbase;
+  if (xcnt < 0) xcnt = 0;
+  const int per_slot = (xcnt + S - 1) / S;
+  const int sbase = qs * per_slot;
+  count = (sbase + per_slot < xcnt ? sbase + per_slot : xcnt) - sbase;
+  if (count < 0) count = 0;
+  first = xbase + sbase;
+}
+__host__ __device__ __forceinline__ int ws_queue_tile(int mode, int first, int idx, int total, int X) {
+  return mode == WS_GLOBAL ? chiplet_transform(idx, total, X) : first + idx;
 }
 
 // Tile id -> (row block, column block).  Column panels of panel_n tiles (the last may be narrower) are
@@ -1069,7 +1106,42 @@ struct Sched {
       // one per queue.
       const int X = p.num_xcds, S = p.counters_per_xcd;
       const int xcd = pid % X, slot = (pid / X) % S;
-      const int per_xcd = (p.total_tiles + X - 1) / X;
+      if (p.ws_mode != WS_QUEUES) {
+        // one queue for everybody, or the XCDs' queues and the shared pool (`step` counts the queues
+        // this workgroup has found empty); an XCD's counter is its slot-0 line, the pool's sits
+        // behind all XCD x slot lines
+        if (tid == 0) {
+          int found = -1;
+          if (p.ws_mode == WS_GLOBAL) {
+            if (step == 0) {
+              const int idx = atomicAdd(p.counters, 1);
+              if (idx < p.total_tiles) found = chiplet_transform(idx, p.total_tiles, X);
+              else step = 1;
+            }
+          } else {
+            // queue order: the own XCD's queue, the shared pool, then the other XCDs' queues (those
+            // only still hold tiles when their own workgroups are masked out or late)
+            while (found < 0 && step <= X) {
+              int line, bound, first;
+              if (step == 1) { line = X * S; bound = p.ws_global; first = X * p.ws_local; }
+              else { const int qx = (xcd + (step == 0 ? 0 : step - 1)) % X; line = qx * S; bound = p.ws_local; first = qx * p.ws_local; }
+              int32_t* ctr = p.counters + line * COUNTER_STRIDE;
+              int idx = bound;
+              if (bound > 0 && __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < bound) idx = atomicAdd(ctr, 1);
+              if (idx < bound) found = first + idx;
+              else ++step;
+            }
+          }
+          s_bcast[0] = found; s_bcast[1] = step;
+        }
+        __syncthreads();
+        const int tile = s_bcast[0];
+        step = s_bcast[1];
+        __syncthreads();
+        if (tile < 0) return false;
+        plain_tile(p, tile, T::BM, T::BN, w.tc);
+        return true;
+      }
       if (tid < 64) {
         const int lane = tid;
         int found = -1, found_step = X * S;
@@ -1078,11 +1150,9 @@ struct Sched {
           const bool valid = v < X * S;
           const int qx = (xcd + v / S) % X;
           const int qs = (slot + v % S) % S;
-          const int xbase = qx * per_xcd;
-          const int xcnt = max(min(xbase + per_xcd, p.total_tiles) - xbase, 0);
-          const int per_slot = (xcnt + S - 1) / S;
-          const int sbase = qs * per_slot;
-          const int bound = valid ? max(min(sbase + per_slot, xcnt) - sbase, 0) : 0;
+          int qfirst, qcount;
+          ws_queue_range(WS_QUEUES, qx * S + qs, p.total_tiles, X, S, 0, qfirst, qcount);
+          const int bound = valid ? qcount : 0;
           int32_t* ctr = p.counters + (qx * S + qs) * COUNTER_STRIDE;
           const int seen = bound > 0 ? __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
           unsigned long long open = __ballot(bound > 0 && seen < bound);
@@ -1091,7 +1161,7 @@ struct Sched {
             int idx = 0;
             if (lane == l) idx = atomicAdd(ctr, 1);
             idx = __shfl(idx, l);
-            const int b = __shfl(bound, l), first = __shfl(xbase + sbase, l);
+            const int b = __shfl(bound, l), first = __shfl(qfirst, l);
             if (idx < b) { found = first + idx; found_step = base + l; }
             open &= open - 1;
           }
@@ -1206,7 +1276,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
     // the last workgroup to leave rearms the queues for the next launch
     uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
     if (done == gridDim.x - 1) {
-      for (int qi = 0; qi < p.num_xcds * p.counters_per_xcd; ++qi)
+      for (int qi = 0; qi <= p.num_xcds * p.counters_per_xcd; ++qi)   // (the last line is the shared pool's)
         __hip_atomic_store(p.counters + qi * COUNTER_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }

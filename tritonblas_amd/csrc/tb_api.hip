@@ -135,6 +135,7 @@ struct Job {
   int schedule = TB_SCHED_PERSISTENT, grid = 0, counters_per_xcd = 0;
   void* workspace = nullptr; size_t workspace_bytes = 0;
   uint32_t epoch = 1, spin_limit = 0;
+  const int32_t* cu_mask = nullptr; int cu_mask_len = 0, ws_mode = 0, ws_local = 0, ws_global = 0;
   // grouped
   const int32_t* group_offsets = nullptr; int num_groups = 0;
   int64_t b_group_stride = 0, sb_group_stride = 0;
@@ -280,10 +281,20 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     { const char* e = getenv("TB_GRID"); if (e && atoi(e) > 0) grid = (int)std::min<int64_t>(total, atoi(e)); }
   } else if (j.schedule == TB_SCHED_WORK_STEALING) {
     p.mode = MODE_WS;
-    grid = j.grid > 0 ? j.grid : resident;
+    grid = j.grid > 0 ? j.grid : (j.cu_mask ? j.cu_mask_len : resident);
+    if (j.cu_mask && (j.cu_mask_len <= 0 || grid > j.cu_mask_len)) return TB_ERR_BAD_ARGUMENT;
+    p.cu_mask = j.cu_mask;
     p.counters_per_xcd = j.counters_per_xcd > 0 ? j.counters_per_xcd : ws_counters_per_xcd(total);
+    p.ws_mode = j.ws_mode;
+    if (j.ws_mode == TB_WS_HIERARCHICAL) {
+      if (j.ws_local < 0 || j.ws_global < 0 || (int64_t)j.ws_local * p.num_xcds + j.ws_global != total) return TB_ERR_BAD_SCHEDULE;
+      p.ws_local = j.ws_local; p.ws_global = j.ws_global;
+    } else if (j.ws_mode != TB_WS_QUEUES && j.ws_mode != TB_WS_GLOBAL_ATOMIC) {
+      return TB_ERR_BAD_SCHEDULE;
+    }
+    // one counter line per XCD x slot, plus the line of the hierarchical mode's shared pool
     plan->ws_counters_off = CTL_WORDS * 4;
-    plan->ws_need = plan->ws_counters_off + (size_t)p.num_xcds * p.counters_per_xcd * COUNTER_STRIDE * 4;
+    plan->ws_need = plan->ws_counters_off + ((size_t)p.num_xcds * p.counters_per_xcd + 1) * COUNTER_STRIDE * 4;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
     int64_t g = j.grid > 0 ? j.grid : streamk_grid(total, p.k_iters, resident);
@@ -352,6 +363,8 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   j->bm = d->block_m; j->bn = d->block_n; j->bk = d->block_k; j->group_m = d->group_m; j->num_xcds = d->num_xcds;
   j->schedule = d->schedule; j->grid = d->grid; j->counters_per_xcd = d->counters_per_xcd;
   j->workspace = d->workspace; j->workspace_bytes = d->workspace_bytes; j->epoch = d->epoch; j->spin_limit = d->spin_limit;
+  j->cu_mask = d->cu_mask; j->cu_mask_len = d->cu_mask_len; j->ws_mode = d->ws_mode;
+  j->ws_local = d->ws_local_tiles_per_xcd; j->ws_global = d->ws_global_tiles;
   return TB_OK;
 }
 
@@ -367,6 +380,22 @@ int tb_tile_coords(int32_t tile, int32_t tiles_m, int32_t tiles_n, int32_t group
   int m, n;
   tile_coords(tile, tiles_m, tiles_n, group_m, panel_n, m, n);
   *pm = m; *pn = n;
+  return TB_OK;
+}
+
+int tb_ws_queue_tile(int32_t ws_mode, int32_t queue, int32_t idx, int32_t total_tiles, int32_t num_xcds,
+                     int32_t counters_per_xcd, int32_t local_tiles_per_xcd, int32_t* count, int32_t* tile) {
+  if (!count || !tile) return TB_ERR_NULL_POINTER;
+  if (ws_mode < TB_WS_QUEUES || ws_mode > TB_WS_HIERARCHICAL || total_tiles <= 0 || num_xcds <= 0 || counters_per_xcd <= 0 ||
+      queue < 0 || idx < 0 || local_tiles_per_xcd < 0)
+    return TB_ERR_BAD_ARGUMENT;
+  const int nq = ws_mode == TB_WS_QUEUES ? num_xcds * counters_per_xcd : ws_mode == TB_WS_GLOBAL_ATOMIC ? 1 : num_xcds + 1;
+  if (queue >= nq) return TB_ERR_BAD_ARGUMENT;
+  if (ws_mode == TB_WS_HIERARCHICAL && (int64_t)local_tiles_per_xcd * num_xcds > total_tiles) return TB_ERR_BAD_ARGUMENT;
+  int first, cnt;
+  ws_queue_range(ws_mode, queue, total_tiles, num_xcds, counters_per_xcd, local_tiles_per_xcd, first, cnt);
+  *count = cnt;
+  *tile = idx < cnt ? ws_queue_tile(ws_mode, first, idx, total_tiles, num_xcds) : -1;
   return TB_OK;
 }
 

@@ -70,6 +70,23 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
         d.group_m, d.num_xcds = selector.group_m, selector.num_sms
         d.counters_per_xcd = selector.COUNTERS_PER_XCD
     d.schedule = schedule
+    if selector is not None and getattr(selector, "_total_cus", None) is not None and schedule != _lib.TB_SCHED_STREAMK:
+        # a selector built for a CU partition sizes the launch (reference matmul.py:113: grid = N_CU):
+        # as many workgroups as that many CUs hold at once; a mask (below) makes it one per mask entry
+        d.grid = selector._N_CU * max(1, selector.waves_per_eu)
+    if schedule == _lib.TB_SCHED_WORK_STEALING and config is not None:
+        # reference matmul.py:112-159: GLOBAL_ATOMIC from the config, the per-workgroup mask by program id
+        if getattr(config, "hierarchical", False) and selector is not None:
+            d.ws_mode = _lib.TB_WS_HIERARCHICAL
+            d.ws_local_tiles_per_xcd, d.ws_global_tiles = selector.hierarchical_split(selector.num_sms)
+        elif config.global_atomic:
+            d.ws_mode = _lib.TB_WS_GLOBAL_ATOMIC
+        mask = config.active_mask()
+        if mask is not None:
+            if mask.dtype != torch.int32 or not mask.is_contiguous() or mask.device != dev:
+                raise RuntimeError("tritonblas_amd: config.mask must be a contiguous int32 tensor on the GEMM's device")
+            d.cu_mask, d.cu_mask_len = _ptr(mask), mask.numel()
+            d.grid = 0
     if schedule == _lib.TB_SCHED_STREAMK:
         if sk_grid is not None:
             d.grid = int(sk_grid)

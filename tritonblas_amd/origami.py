@@ -73,6 +73,7 @@ class OrigamiMatmulSelector:
         if total_cus is not None:
             self._hardware.N_CU = total_cus
             self._hardware._c.n_cu = total_cus
+        self._total_cus = total_cus
         self._N_CU = self._hardware.N_CU
         self._ACTIVE_CU = active_cus if active_cus is not None else self._N_CU
         self._active_cus = active_cus
@@ -98,6 +99,22 @@ class OrigamiMatmulSelector:
     waves_per_eu = property(lambda self: self._sel.occupancy)
     sk_grid = property(lambda self: self._grid)
     estimate_us = property(lambda self: self._sel.est_total_us)
+
+    def hierarchical_split(self, num_xcds: int) -> tuple:
+        """(local_tiles_per_xcd, global_tiles) of the hierarchical work-stealing mode (reference
+        origami.py:288-311): up to 4 tiles per CU everything is XCD-local; above that the local share
+        falls by 5 % per extra tile per CU down to one half, the rest goes to the pool every XCD
+        steals from.  Uses the hardware CU count, not the active one.  Where the reference's formula
+        hands out more local tiles than there are (fewer tiles than XCDs), the local queues get what
+        divides evenly instead."""
+        bm, bn = self.block_m, self.block_n
+        total_tiles = ((self._m + bm - 1) // bm) * ((self._n + bn - 1) // bn)
+        hw_cus = self._hardware._c.num_xcd * self._hardware._c.cu_per_xcd
+        tiles_per_cu = total_tiles / max(hw_cus, 1)
+        local_frac = max(0.5, 1.0 - max(0.0, tiles_per_cu - 4.0) * 0.05)
+        local_per_xcd = max(int(total_tiles * local_frac) // num_xcds, 1)
+        local_per_xcd = min(local_per_xcd, total_tiles // num_xcds)
+        return local_per_xcd, total_tiles - local_per_xcd * num_xcds
 
     @property
     def even_k(self):
