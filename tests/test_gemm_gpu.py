@@ -353,6 +353,80 @@ def test_skinny_rows(m, n, k, dtype):
         _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32, bias=bias), dtype, TOL_16)
 
 
+# ---- fp32 operands ------------------------------------------------------------------------------
+TOL_32 = 1e-5   # full fp32 products and sums; a TF32-style 10-bit mantissa would sit near 5e-4
+
+
+def _ref64(a_cpu, b_cpu, bias=None):
+    acc = torch.matmul(a_cpu.double(), b_cpu.double())
+    return acc if bias is None else acc + bias.double()[None, :]
+
+
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (512, 768, 320), (300, 200, 192), (257, 129, 67), (16, 2048, 512),
+                                   (2048, 64, 4096), (1, 1, 1)])
+@pytest.mark.parametrize("transA,transB", [("T", "T"), ("N", "N"), ("T", "N"), ("N", "T")])
+def test_matmul_fp32(m, n, k, transA, transB):
+    """float32 in, float32 out (reference tests/test_matmul.py:23): K-contiguous operands run the
+    LDS-direct kernels, every other layout the gather kernel."""
+    import tritonblas_amd as tb
+    _say(f"matmul fp32 {m}x{n}x{k} {transA}{transB}")
+    a_cpu, b_cpu = _rand((m, k), torch.float32, 40, 0.5), _rand((k, n), torch.float32, 41, 0.5)
+    a, b = _layout(a_cpu, transA), _layout(b_cpu, transB)
+    c = tb.matmul(a, b)
+    assert c.shape == (m, n) and c.dtype == torch.float32
+    err = OG.rel_fro_error(c.cpu().double(), _ref64(a_cpu, b_cpu))
+    assert err <= TOL_32, f"relative Frobenius error {err:.3e}"
+
+
+@pytest.mark.parametrize("tile", [(256, 256, 32), (128, 128, 32), (64, 64, 32)])
+@pytest.mark.parametrize("mode", ["persistent", "streamk", "work_stealing"])
+def test_every_fp32_tile_variant_and_schedule(tile, mode):
+    import tritonblas_amd as tb
+    m, n, k = 640, 768, 1024
+    _say(f"matmul_lt fp32 tile={tile} {mode}")
+    a_cpu, b_cpu = _rand((m, k), torch.float32, 42, 0.5), _rand((k, n), torch.float32, 43, 0.5)
+    a, b = a_cpu.cuda(), b_cpu.cuda().T.contiguous().T     # both K-contiguous
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, a.dtype, a.dtype, a.device, streamk=mode == "streamk")
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = tile
+    cfg = tb.matmul_preamble(sel)
+    for rep in range(2):
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        tb.matmul_lt(a, b, c, sel, cfg, enable_streamk=mode == "streamk", work_stealing=mode == "work_stealing")
+        err = OG.rel_fro_error(c.cpu().double(), _ref64(a_cpu, b_cpu))
+        assert err <= TOL_32, f"relative Frobenius error {err:.3e} (launch {rep})"
+
+
+def test_fp32_products_are_not_truncated():
+    """Operands whose low mantissa bits carry the whole answer: (1 + e) * (1 - e) summed against -1."""
+    import tritonblas_amd as tb
+    k = 256
+    e = 2.0 ** -12
+    a = torch.full((64, k), 1.0 + e, dtype=torch.float32)
+    b = torch.full((k, 64), 1.0 - e, dtype=torch.float32)
+    c = tb.matmul(a.cuda(), b.cuda().T.contiguous().T).cpu()
+    want = k * (1.0 - e * e)            # exact in fp32 arithmetic up to the final roundings
+    assert torch.allclose(c, torch.full_like(c, want), rtol=0, atol=k * 2.0 ** -24 * 4)
+    assert abs(float(c[0, 0]) - k) > k * e * e * 0.5   # a 10-bit-mantissa product would return exactly k
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_addmm_fp32(out_dtype):
+    import tritonblas_amd as tb
+    m, n, k = 384, 520, 264
+    a_cpu, b_cpu, bias = _rand((m, k), torch.float32, 44, 0.5), _rand((k, n), torch.float32, 45, 0.5), _rand((n,), torch.float32, 46)
+    if out_dtype == torch.float32:
+        c = tb.addmm(bias.cuda(), a_cpu.cuda(), b_cpu.cuda())
+    else:
+        sel = tb.OrigamiMatmulSelector(m, n, k, torch.float32, torch.float32, out_dtype, torch.device("cuda"))
+        c = torch.zeros(m, n, dtype=out_dtype, device="cuda")
+        from tritonblas_amd.matmul import _launch_gemm
+        from tritonblas_amd import _lib
+        _launch_gemm(a_cpu.cuda(), b_cpu.cuda(), c, sel, None, _lib.TB_SCHED_PERSISTENT, bias=bias.cuda())
+    want = _ref64(a_cpu, b_cpu, bias)
+    err = OG.rel_fro_error(c.cpu().double(), want.to(out_dtype).double())
+    assert err <= (TOL_32 if out_dtype == torch.float32 else TOL_16), f"{err:.3e}"
+
+
 # ---- MXFP4 --------------------------------------------------------------------------------------
 def _fp4_case(m, n, k, seed):
     rng = np.random.default_rng(seed)

@@ -36,7 +36,7 @@ _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "float16": torch.flo
 def str_to_dtype(name):
     key = str(name).replace("torch.", "").lower()
     if key not in _DTYPES:
-        raise ValueError(f"unsupported dtype {name!r}; this library runs float16, bfloat16, float8_e4m3fn and fp4 inputs")
+        raise ValueError(f"unsupported dtype {name!r}; this library runs float32, float16, bfloat16, float8_e4m3fn and fp4 inputs")
     return _DTYPES[key]
 
 

@@ -89,7 +89,7 @@ struct Tile {
   static constexpr bool FAST = FAST_;
   static constexpr bool DMA = USE_DMA_ && FAST && ALAY == LAY_K && BLAY == LAY_K;  // global -> LDS without registers
   static constexpr int THREADS = WM * WN * 64;
-  static constexpr int USZ = (DT == DT_F16 || DT == DT_BF16) ? 2 : 1;  // bytes per storage unit
+  static constexpr int USZ = (DT == DT_F16 || DT == DT_BF16) ? 2 : (DT == DT_F32 ? 4 : 1);  // bytes per storage unit
   static constexpr int UPC = 16 / USZ;                                 // units per 16-byte chunk
   static constexpr int CPR = BKB / 16;                                 // chunks per tile row
   static constexpr int UPS = CPR * UPC;                                // units per K step
@@ -206,7 +206,13 @@ __host__ __device__ __forceinline__ void tile_coords(int tile, int tiles_m, int 
 template <class T>
 __device__ __forceinline__ v4i gather_units(const uint8_t* rowp, int64_t ku, int64_t s_k, int64_t KU) {
   uint32_t w[4] = {0u, 0u, 0u, 0u};
-  if constexpr (T::USZ == 2) {
+  if constexpr (T::USZ == 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      int64_t k = ku + u;
+      w[u] = (k < KU) ? *(const uint32_t*)(rowp + k * s_k * 4) : 0u;
+    }
+  } else if constexpr (T::USZ == 2) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       int64_t k = ku + u;
@@ -406,6 +412,15 @@ __device__ __forceinline__ v4f mma(typename Frag<T>::type x, typename Frag<T>::t
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, x), __builtin_bit_cast(h8, y), c, 0, 0, 0);
   } else if constexpr (T::DT == DT_BF16) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, x), __builtin_bit_cast(bf8, y), c, 0, 0, 0);
+  } else if constexpr (T::DT == DT_F32) {
+    // four 16x16x4 steps: lane group g feeds k = 4g + i to step i (any assignment works as long as
+    // both operands use the same one), so one 16-byte fragment is consumed without shuffles
+    // (reinterpret the whole vectors: a bit cast of one vector *element* reads element 0 with this compiler)
+    const v4f xf = __builtin_bit_cast(v4f, x), yf = __builtin_bit_cast(v4f, y);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[0], yf[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[1], yf[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[2], yf[2], c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(xf[3], yf[3], c, 0, 0, 0);
   } else if constexpr (T::DT == DT_FP8) {
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
   } else {

@@ -29,5 +29,7 @@ extern const Variant g_variants_fp8[];
 extern const int g_num_variants_fp8;
 extern const Variant g_variants_fp4[];
 extern const int g_num_variants_fp4;
+extern const Variant g_variants_f32[];
+extern const int g_num_variants_f32;
 
 }  // namespace tb

@@ -71,6 +71,7 @@ void variant_table(int dt, const Variant** v, int* n) {
     case TB_BF16: *v = g_variants_bf16; *n = g_num_variants_bf16; break;
     case TB_FP8_E4M3: *v = g_variants_fp8; *n = g_num_variants_fp8; break;
     case TB_FP4_E2M1: *v = g_variants_fp4; *n = g_num_variants_fp4; break;
+    case TB_F32: *v = g_variants_f32; *n = g_num_variants_f32; break;
     default: *v = nullptr; *n = 0;
   }
 }
@@ -117,7 +118,7 @@ int default_panel_n(int grid, int chunk, int group_m) {
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
-int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : 1; }
+int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : (dt == TB_F32 ? 4 : 1); }
 int c_bytes(int t) { return t == TB_F32 ? 4 : 2; }
 
 // Everything the launch path needs, independent of which public descriptor it came from.
@@ -351,7 +352,7 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
   if (d->a_type != d->b_type) return TB_ERR_BAD_DTYPE;
-  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3) return TB_ERR_BAD_DTYPE;
+  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_F32) return TB_ERR_BAD_DTYPE;
   if ((d->a_scale == nullptr) != (d->b_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
   if (d->bias && d->bias_type != TB_F16 && d->bias_type != TB_BF16 && d->bias_type != TB_F32) return TB_ERR_BAD_DTYPE;
   j->dt = d->a_type; j->c_type = d->c_type; j->bias_type = d->bias_type;
