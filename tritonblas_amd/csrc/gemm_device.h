@@ -1106,9 +1106,11 @@ struct Sched {
       return true;
     }
     if (p.mode == MODE_GROUPED) {
-      if (next_tile < 0) return false;
+      // the grid loops over the tile table; the first id past the table's end finishes the workgroup
+      // (the host only knows an upper bound of the table's length)
+      if (next_tile >= p.total_tiles) return false;
       bool ok = grouped_tile(p, next_tile, T::BM, T::BN, T::USZ, w.tc);
-      next_tile = -1;
+      next_tile = ok ? next_tile + G : p.total_tiles;
       return ok;
     }
     if (p.mode == MODE_WS) {

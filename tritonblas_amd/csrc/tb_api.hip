@@ -273,8 +273,14 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   int grid;
   plan->ws_need = 0;
   if (j.num_groups > 0) {
+    // the tile table has at most this many entries (every expert may end in a partial row block);
+    // a resident grid loops over it
     p.mode = MODE_GROUPED;
-    grid = (int)(((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n);
+    const int64_t bound = ((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n;
+    if (bound > INT32_MAX) return TB_ERR_BAD_SHAPE;
+    p.total_tiles = (int32_t)bound;
+    grid = (int)std::min<int64_t>(bound, resident);
+    { const char* e = getenv("TB_GRID"); if (e && atoi(e) > 0) grid = (int)std::min<int64_t>(bound, atoi(e)); }
   } else if (j.schedule == TB_SCHED_PERSISTENT) {
     // a resident grid that loops over the tiles (matmul.py:160-198: for tile_id in range(pid, total, NUM_SMS))
     p.mode = MODE_STATIC;
