@@ -139,8 +139,9 @@ typedef struct tb_gemm_desc {
                                  (the reference launches one per CU and masks by program id)          */
   int32_t cu_mask_len;
   int32_t ws_mode;            /* TB_WS_*                                                            */
-  int32_t ws_local_tiles_per_xcd, ws_global_tiles;  /* TB_WS_HIERARCHICAL: num_xcds * local + global
-                                 must equal the tile count                                           */
+  int32_t ws_local_tiles_per_xcd, ws_global_tiles;  /* TB_WS_HIERARCHICAL: both 0 = split by the
+                                 reference's rule (tb_hierarchical_split) for the tile the launch
+                                 runs; otherwise num_xcds * local + global must equal its tile count */
 } tb_gemm_desc;
 
 /* C = cast((A @ B) * a_scale[:,None] * b_scale[None,:] + bias[None,:]), fp32 accumulate.
@@ -215,6 +216,11 @@ int tb_hadamard_mxfp4_quant(const tb_quant_desc* desc, void* stream);
  * tb_default_panel gives the panel width tb_gemm uses for a launch grid. */
 int tb_tile_coords(int32_t tile, int32_t tiles_m, int32_t tiles_n, int32_t group_m, int32_t panel_n, int32_t* pm, int32_t* pn);
 int tb_default_panel(int32_t grid, int32_t chunk, int32_t group_m);
+
+/* (tiles per XCD-local queue, tiles in the shared pool) for total_tiles tiles on hw_cus compute units
+ * (the hardware count, not the active one) and num_xcds queues: hierarchical_split, origami.py:288-311;
+ * the local share is capped at what divides evenly, so the two always add up to total_tiles. */
+int tb_hierarchical_split(int64_t total_tiles, int32_t hw_cus, int32_t num_xcds, int32_t* local_tiles_per_xcd, int32_t* global_tiles);
 
 /* Host-side evaluation of the work-stealing queues: queue `queue` of a launch over total_tiles tiles
  * (TB_WS_QUEUES: queue = xcd * counters_per_xcd + slot; TB_WS_GLOBAL_ATOMIC: queue 0;

@@ -351,3 +351,19 @@ def test_matmul_config_mask_rules():
     assert cfg.active_mask() is None
     cfg2 = MatmulConfig(device=torch.device("cpu"), workspace=None, mask=m, use_mask=False)   # what matmul_preamble does with all CUs active
     assert cfg2.mask is m and cfg2.active_mask() is None
+
+
+@pytest.mark.parametrize("total", [1, 5, 8, 9, 63, 512, 1024, 1100, 2048, 3584, 5120, 100000])
+@pytest.mark.parametrize("hw_cus,xcds", [(256, 8), (304, 8), (64, 4), (32, 1)])
+def test_library_hierarchical_split(total, hw_cus, xcds):
+    lib = _load()
+    l, g = C.c_int32(), C.c_int32()
+    assert lib.tb_hierarchical_split(total, hw_cus, xcds, C.byref(l), C.byref(g)) == 0
+    want = OS.hierarchical_split(total, hw_cus, xcds)
+    assert l.value * xcds + g.value == total and l.value >= 0 and g.value >= 0
+    if want[1] >= 0:
+        assert (l.value, g.value) == want
+    else:
+        assert (l.value, g.value) == (total // xcds, total - xcds * (total // xcds))
+    assert lib.tb_hierarchical_split(0, hw_cus, xcds, C.byref(l), C.byref(g)) == -10
+    assert lib.tb_hierarchical_split(total, hw_cus, xcds, None, C.byref(g)) == -1

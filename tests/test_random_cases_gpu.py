@@ -1,0 +1,89 @@
+"""Seeded random sweep over the GEMM entry points: element type x operand layouts x schedule x odd
+shapes (any M, N, K including non-multiples of the vector width, slices with a row pitch), against
+the CPU oracle.  Every launch goes through the C ABI.  TB_RANDOM_CASES / TB_RANDOM_SEED widen the sweep."""
+import os
+import random
+import sys
+
+import pytest
+import torch
+
+from oracle import gemm as OG
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: 1e-3, torch.bfloat16: 1e-3, torch.float32: 1e-5, torch.float8_e4m3fn: 1e-2}
+
+
+def _cases(n, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        dtype = rng.choice([torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn])
+        big = rng.random() < 0.3
+        m = rng.randint(1, 1500 if big else 300)
+        nn = rng.randint(1, 1500 if big else 300)
+        k = rng.choice([rng.randint(1, 2048), 32 * rng.randint(1, 64), 128 * rng.randint(1, 24)])
+        out.append(dict(idx=i, dtype=dtype, m=m, n=nn, k=k, ta=rng.choice("TN"), tb=rng.choice("TN"),
+                        sched=rng.choice(["persistent", "streamk", "ws", "ws_global", "ws_hier"]),
+                        pitch=rng.choice([0, 0, 8, 3]), bias=rng.random() < 0.3, seed=rng.randint(0, 1 << 30)))
+    return out
+
+
+def _place(x_cpu, trans, pitch):
+    """'T': the logical matrix is contiguous; 'N': its transpose is.  pitch > 0: rows sit in a wider buffer."""
+    x = x_cpu.cuda()
+    if trans == "N":
+        x = x.T
+    rows, cols = x.shape
+    buf = torch.zeros(rows, cols + pitch, dtype=torch.uint8 if x.dtype == torch.float8_e4m3fn else x.dtype, device="cuda")
+    if x.dtype == torch.float8_e4m3fn:
+        buf = buf.view(torch.float8_e4m3fn)
+        buf.view(torch.uint8)[:, :cols] = x.contiguous().view(torch.uint8)
+    else:
+        buf[:, :cols] = x
+    v = buf[:, :cols]
+    return v.T if trans == "N" else v
+
+
+@pytest.mark.parametrize("case", _cases(int(os.environ.get("TB_RANDOM_CASES", "72")), int(os.environ.get("TB_RANDOM_SEED", "20241"))), ids=lambda c: f"{c['idx']}-{str(c['dtype']).split('.')[-1]}-{c['m']}x{c['n']}x{c['k']}-{c['ta']}{c['tb']}-{c['sched']}")
+def test_random_case(case):
+    import tritonblas_amd as tb
+    print("random case", case, flush=True)
+    sys.stdout.flush()
+    dtype, m, n, k = case["dtype"], case["m"], case["n"], case["k"]
+    g = torch.Generator().manual_seed(case["seed"])
+    a32, b32 = torch.randn(m, k, generator=g) * 0.5, torch.randn(k, n, generator=g) * 0.5
+    quant = dtype == torch.float8_e4m3fn
+    out_dtype = torch.bfloat16 if quant else dtype
+    bias = (torch.randn(n, generator=g).to(out_dtype) if case["bias"] and not quant else None)
+    if quant:
+        a_cpu, sa = OG.quantize_per_channel_fp8(a32, axis=1)
+        b_cpu, sb = OG.quantize_per_channel_fp8(b32, axis=0)
+    else:
+        a_cpu, b_cpu, sa, sb = a32.to(dtype), b32.to(dtype), None, None
+    a, b = _place(a_cpu, case["ta"], case["pitch"]), _place(b_cpu, case["tb"], case["pitch"])
+    assert a.shape == (m, k) and b.shape == (k, n)
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, out_dtype, a.device, streamk=case["sched"] == "streamk")
+    cfg = tb.matmul_preamble(sel)
+    cfg.global_atomic, cfg.hierarchical = case["sched"] == "ws_global", case["sched"] == "ws_hier"
+    ws, sk = case["sched"].startswith("ws"), case["sched"] == "streamk"
+    c = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+    if quant:
+        tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, cfg, enable_streamk=sk, work_stealing=ws)
+    elif bias is not None:
+        from tritonblas_amd import _lib
+        from tritonblas_amd.matmul import _launch_gemm
+        sched = _lib.TB_SCHED_STREAMK if sk else (_lib.TB_SCHED_WORK_STEALING if ws else _lib.TB_SCHED_PERSISTENT)
+        _launch_gemm(a, b, c, sel, cfg, sched, bias=bias.cuda())
+    else:
+        tb.matmul_lt(a, b, c, sel, cfg, enable_streamk=sk, work_stealing=ws)
+    want = torch.matmul(a_cpu.double(), b_cpu.double())
+    if quant:
+        want = want * (sa.double()[:, None] * sb.double()[None, :])
+    if bias is not None:
+        want = want + bias.double()[None, :]
+    got = c.cpu()
+    assert torch.isfinite(got.float()).all(), "unwritten or non-finite outputs"
+    err = OG.rel_fro_error(got.double(), want.float().to(out_dtype).double())
+    assert err <= TOL[dtype], f"relative Frobenius error {err:.3e} > {TOL[dtype]}"

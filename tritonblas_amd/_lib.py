@@ -23,7 +23,7 @@ TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
 EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
-    "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile",
+    "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile", "tb_hierarchical_split",
 ]
 
 
@@ -116,6 +116,7 @@ def load():
     lib.tb_tile_coords.argtypes = [C.c_int32] * 5 + [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.tb_default_panel.argtypes = [C.c_int32] * 3
     lib.tb_ws_queue_tile.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32)] * 2
+    lib.tb_hierarchical_split.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     if lib.tb_abi_version() != 1:
         raise RuntimeError("libtritonblas_amd.so ABI version mismatch")
     _lib = lib

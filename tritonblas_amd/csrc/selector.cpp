@@ -44,6 +44,19 @@ int ws_counters_per_xcd(int64_t total_tiles) {
   return 1;
 }
 
+// Reference origami.py:288-311: up to 4 tiles per CU everything stays XCD-local; above that the local
+// share falls by 5 % per extra tile per CU, down to one half.  The local queues never get more than
+// divides evenly (the reference's formula hands out one tile per XCD even when there are fewer tiles
+// than XCDs).
+void hierarchical_split(int64_t total_tiles, int hw_cus, int num_xcds, int64_t* local_per_xcd, int64_t* global_tiles) {
+  const double tiles_per_cu = (double)total_tiles / std::max(hw_cus, 1);
+  const double local_frac = std::max(0.5, 1.0 - std::max(0.0, tiles_per_cu - 4.0) * 0.05);
+  int64_t local = std::max<int64_t>((int64_t)((double)total_tiles * local_frac) / num_xcds, 1);
+  local = std::min(local, total_tiles / num_xcds);
+  *local_per_xcd = local;
+  *global_tiles = total_tiles - local * num_xcds;
+}
+
 static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Workgroups of one variant that fit a CU (LDS and wave slots), capped by what the kernel was built for.

@@ -294,8 +294,10 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     p.counters_per_xcd = j.counters_per_xcd > 0 ? j.counters_per_xcd : ws_counters_per_xcd(total);
     p.ws_mode = j.ws_mode;
     if (j.ws_mode == TB_WS_HIERARCHICAL) {
-      if (j.ws_local < 0 || j.ws_global < 0 || (int64_t)j.ws_local * p.num_xcds + j.ws_global != total) return TB_ERR_BAD_SCHEDULE;
-      p.ws_local = j.ws_local; p.ws_global = j.ws_global;
+      int64_t local = j.ws_local, global = j.ws_global;
+      if (local == 0 && global == 0) hierarchical_split(total, hw.num_xcd * hw.cu_per_xcd, p.num_xcds, &local, &global);
+      if (local < 0 || global < 0 || local * p.num_xcds + global != total) return TB_ERR_BAD_SCHEDULE;
+      p.ws_local = (int32_t)local; p.ws_global = (int32_t)global;
     } else if (j.ws_mode != TB_WS_QUEUES && j.ws_mode != TB_WS_GLOBAL_ATOMIC) {
       return TB_ERR_BAD_SCHEDULE;
     }
@@ -403,6 +405,15 @@ int tb_ws_queue_tile(int32_t ws_mode, int32_t queue, int32_t idx, int32_t total_
   ws_queue_range(ws_mode, queue, total_tiles, num_xcds, counters_per_xcd, local_tiles_per_xcd, first, cnt);
   *count = cnt;
   *tile = idx < cnt ? ws_queue_tile(ws_mode, first, idx, total_tiles, num_xcds) : -1;
+  return TB_OK;
+}
+
+int tb_hierarchical_split(int64_t total_tiles, int32_t hw_cus, int32_t num_xcds, int32_t* local_tiles_per_xcd, int32_t* global_tiles) {
+  if (!local_tiles_per_xcd || !global_tiles) return TB_ERR_NULL_POINTER;
+  if (total_tiles <= 0 || total_tiles > INT32_MAX || hw_cus <= 0 || num_xcds <= 0) return TB_ERR_BAD_ARGUMENT;
+  int64_t l, g;
+  hierarchical_split(total_tiles, hw_cus, num_xcds, &l, &g);
+  *local_tiles_per_xcd = (int32_t)l; *global_tiles = (int32_t)g;
   return TB_OK;
 }
 

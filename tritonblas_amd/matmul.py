@@ -76,9 +76,10 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
         d.grid = selector._N_CU * max(1, selector.waves_per_eu)
     if schedule == _lib.TB_SCHED_WORK_STEALING and config is not None:
         # reference matmul.py:112-159: GLOBAL_ATOMIC from the config, the per-workgroup mask by program id
-        if getattr(config, "hierarchical", False) and selector is not None:
+        if getattr(config, "hierarchical", False):
+            # (the split is left to the library: it knows the tile the launch really runs, which is not
+            # the selector's when the operands need the gather kernel)
             d.ws_mode = _lib.TB_WS_HIERARCHICAL
-            d.ws_local_tiles_per_xcd, d.ws_global_tiles = selector.hierarchical_split(selector.num_sms)
         elif config.global_atomic:
             d.ws_mode = _lib.TB_WS_GLOBAL_ATOMIC
         mask = config.active_mask()

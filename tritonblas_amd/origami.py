@@ -110,11 +110,10 @@ class OrigamiMatmulSelector:
         bm, bn = self.block_m, self.block_n
         total_tiles = ((self._m + bm - 1) // bm) * ((self._n + bn - 1) // bn)
         hw_cus = self._hardware._c.num_xcd * self._hardware._c.cu_per_xcd
-        tiles_per_cu = total_tiles / max(hw_cus, 1)
-        local_frac = max(0.5, 1.0 - max(0.0, tiles_per_cu - 4.0) * 0.05)
-        local_per_xcd = max(int(total_tiles * local_frac) // num_xcds, 1)
-        local_per_xcd = min(local_per_xcd, total_tiles // num_xcds)
-        return local_per_xcd, total_tiles - local_per_xcd * num_xcds
+        local, pool = _lib.C.c_int32(), _lib.C.c_int32()
+        _lib.check(_lib.load().tb_hierarchical_split(total_tiles, hw_cus, int(num_xcds), _lib.C.byref(local), _lib.C.byref(pool)),
+                   "tb_hierarchical_split")
+        return local.value, pool.value
 
     @property
     def even_k(self):
