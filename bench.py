@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp4": 10100.0}
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp4": 10100.0, "fp32": 157.3}
 PEAK_HBM_GBPS = 8000.0
 
 
@@ -180,6 +180,16 @@ def main():
         sec["bf16_gemm_8192x8192x8192_TN"] = {"ms": round(bms, 4), "TFLOP/s": round(tf2, 1),
                                               "frac_mfma_peak": round(tf2 / PEAK_TFLOPS["bf16"], 4)}
         del a2, b2, c2
+        # fp32 TN 8192^3 (16x16x4 fp32 MFMA: full fp32 products)
+        a3 = (torch.rand(8192, 8192, device=dev, generator=g) * 2 - 1)
+        b3 = (torch.rand(8192, 8192, device=dev, generator=g) * 2 - 1).T
+        c3 = torch.empty(8192, 8192, dtype=torch.float32, device=dev)
+        sel3 = tb.OrigamiMatmulSelector(8192, 8192, 8192, a3.dtype, b3.dtype, c3.dtype, dev)
+        f32ms, _ = timed(lambda: tb.matmul_lt(a3, b3, c3, sel3, None), max(5, steps2 // 2), 2)
+        tf3 = 2.0 * 8192 ** 3 / f32ms / 1e9
+        sec["fp32_gemm_8192x8192x8192_TN"] = {"ms": round(f32ms, 4), "TFLOP/s": round(tf3, 1),
+                                              "frac_mfma_peak": round(tf3 / PEAK_TFLOPS["fp32"], 4)}
+        del a3, b3, c3
         # FP8 decode: the library routes M <= 64 to its streaming kernel (weight read once, split-K inside the workgroup)
         Md, Nd, Kd = 32, 8192, 28672
         aqd, wqd, sad, swd = fp8_inputs(Md, Nd, Kd, dev, 22)
