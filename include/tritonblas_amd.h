@@ -41,7 +41,9 @@ enum {
   TB_BF16 = 1,
   TB_FP8_E4M3 = 2,  /* OCP e4m3fn                                                  */
   TB_FP4_E2M1 = 3,  /* two codes per byte, low nibble = even k (utils.py:585-587) */
-  TB_F32 = 4        /* operands (full fp32 products, 16x16x4 MFMA), output, bias, quantiser input */
+  TB_F32 = 4,       /* operands (full fp32 products, 16x16x4 MFMA), output, bias, quantiser input */
+  TB_I8 = 5         /* operands (int32 sums, persistent_gemm.py:75); as output only with TB_I8 operands: fp32 epilogue
+                       result truncated toward zero and saturated to [-128, 127]                    */
 };
 
 /* ---- schedules ------------------------------------------------------------------------------ */

@@ -26,6 +26,33 @@ def quantize_per_channel_fp8(x: torch.Tensor, axis: int, dtype=torch.float8_e4m3
     return q, scale.squeeze(axis).to(torch.float32)
 
 
+def quantize_per_channel_int8(x: torch.Tensor, axis: int, min_scale: float = 1e-8):
+    """include/tritonblas/utils.py:364-375, int8 branch: amax -> scale = amax/127 ->
+    q = clamp(round(x * (1/scale)), -127, 127).to(int8)."""
+    base = x.to(torch.float32)
+    max_abs = torch.clamp(base.abs().amax(dim=axis, keepdim=True), min=min_scale)
+    scale = max_abs / 127.0
+    q = torch.round(base * (1.0 / scale)).clamp_(-127.0, 127.0).to(torch.int8)
+    return q, scale.squeeze(axis).to(torch.float32)
+
+
+def ref_gemm_int8(a: torch.Tensor, b: torch.Tensor, out_dtype, a_scale=None, b_scale=None, bias=None):
+    """int8 operands: exact integer sums (include/tritonblas/kernels/persistent_gemm.py:75), then the
+    a8w8 epilogue in fp32 (tests/test_matmul_a8w8_lt.py:11-38).  out_dtype int8: the fp32 result is
+    truncated toward zero and saturated to [-128, 127] -- a decision of this build: the reference
+    converts with a bare float->int8 cast, which is undefined outside that range, its own (switched
+    off) test clamps the expectation to +-127 and compares at atol 5; parity unpinned.
+    Returns fp64 for float out types (the caller rounds) and int8 for int8."""
+    acc = torch.matmul(a.to(torch.int64), b.to(torch.int64)).to(torch.float64)
+    if a_scale is not None and b_scale is not None:
+        acc = (acc.to(torch.float32) * (a_scale.to(torch.float32)[:, None] * b_scale.to(torch.float32)[None, :])).to(torch.float64)
+    if bias is not None:
+        acc = acc + bias.to(torch.float64)[None, :]
+    if out_dtype == torch.int8:
+        return torch.clamp(torch.trunc(acc.to(torch.float32)), -128, 127).to(torch.int8)
+    return acc
+
+
 def ref_gemm(a: torch.Tensor, b: torch.Tensor, out_dtype=None, a_scale=None, b_scale=None, bias=None):
     """C = cast((fp32(A) @ fp32(B)) * (sa[:,None]*sb[None,:]) + bias[None,:]).
 

@@ -33,8 +33,9 @@ def test_dtype_names():
     from tritonblas_amd.benchmarks.matmul_bench import str_to_dtype
     assert str_to_dtype("bfloat16") is torch.bfloat16 and str_to_dtype("torch.float8_e4m3fn") is torch.float8_e4m3fn
     assert str_to_dtype("fp4") == "fp4"
+    assert str_to_dtype("int8") is torch.int8 and str_to_dtype("float32") is torch.float32
     with pytest.raises(ValueError):
-        str_to_dtype("int8")
+        str_to_dtype("float64")
 
 
 @pytest.mark.gpu
@@ -46,6 +47,9 @@ def test_driver_runs_a_shape_list_with_correctness_check(tmp_path, flags):
         {"m": 256, "n": 512, "k": 1024, "in_dtype": "bfloat16", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
         {"m": 300, "n": 200, "k": 512, "in_dtype": "float16", "out_dtype": "float16", "transA": "T", "transB": "T"},
         {"m": 512, "n": 256, "k": 2048, "in_dtype": "float8_e4m3fn", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+        {"m": 384, "n": 256, "k": 1024, "in_dtype": "int8", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+        {"m": 256, "n": 384, "k": 512, "in_dtype": "int8", "out_dtype": "int8", "transA": "T", "transB": "N"},
+        {"m": 320, "n": 256, "k": 768, "in_dtype": "float32", "out_dtype": "float32", "transA": "T", "transB": "T"},
     ]
     if not flags:
         cases.append({"m": 128, "n": 256, "k": 1024, "in_dtype": "fp4", "out_dtype": "bfloat16", "transA": "T", "transB": "N"})

@@ -427,6 +427,70 @@ def test_addmm_fp32(out_dtype):
     assert err <= (TOL_32 if out_dtype == torch.float32 else TOL_16), f"{err:.3e}"
 
 
+# ---- int8 operands -------------------------------------------------------------------------------
+def _int8_case(m, n, k, seed):
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(seed))
+    b = torch.randn(k, n, generator=torch.Generator().manual_seed(seed + 10000))
+    aq, sa = OG.quantize_per_channel_int8(a, axis=1)
+    bq, sb = OG.quantize_per_channel_int8(b, axis=0)
+    return aq, bq, sa, sb
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (1024, 1024, 1024), (300, 200, 192), (257, 129, 67), (32, 2048, 4096), (1, 1, 1)])
+@pytest.mark.parametrize("transA,transB", [("T", "N"), ("T", "T"), ("N", "N"), ("N", "T")])
+def test_matmul_a8w8_int8_to_bf16(m, n, k, transA, transB):
+    """int8 x int8 with per-row / per-column scales into bf16 (reference persistent_gemm.py:75 with a
+    non-int8 C; the reference's own int8 test is switched off, tests/test_matmul_a8w8_lt.py:62)."""
+    import tritonblas_amd as tb
+    _say(f"a8w8 int8 {m}x{n}x{k} {transA}{transB}")
+    aq, bq, sa, sb = _int8_case(m, n, k, 50)
+    a, b = _layout(aq, transA), _layout(bq, transB)
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
+    tb.matmul_a8w8(a, b, sa.cuda(), sb.cuda(), c)
+    want = OG.ref_gemm_int8(aq, bq, torch.bfloat16, a_scale=sa, b_scale=sb)
+    _check(c.cpu(), want.float(), torch.bfloat16, TOL_16)   # integer sums are exact: only the bf16 rounding is left
+
+
+@pytest.mark.parametrize("tile", [(256, 256, 128), (128, 128, 128), (64, 64, 128)])
+@pytest.mark.parametrize("mode", ["persistent", "streamk", "work_stealing"])
+def test_int8_sums_are_exact_in_every_tile_and_schedule(tile, mode):
+    """No scales, fp32 out: every output is an integer below 2^24 and must come out exactly."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    from tritonblas_amd.matmul import _launch_gemm
+    m, n, k = 640, 768, 1024
+    _say(f"int8 exact tile={tile} {mode}")
+    g = torch.Generator().manual_seed(51)
+    aq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    bq = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int8)
+    want = torch.matmul(aq.to(torch.int64), bq.to(torch.int64).T)
+    assert int(want.abs().max()) < 2 ** 24
+    sel = tb.OrigamiMatmulSelector(m, n, k, torch.int8, torch.int8, torch.float32, torch.device("cuda"), streamk=mode == "streamk")
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = tile
+    cfg = tb.matmul_preamble(sel)
+    sched = {"persistent": _lib.TB_SCHED_PERSISTENT, "streamk": _lib.TB_SCHED_STREAMK, "work_stealing": _lib.TB_SCHED_WORK_STEALING}[mode]
+    for rep in range(2):
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        _launch_gemm(aq.cuda(), bq.cuda().T, c, sel, cfg, sched)
+        assert torch.equal(c.cpu().to(torch.int64), want), f"launch {rep}"
+
+
+def test_int8_output_truncates_and_saturates():
+    import tritonblas_amd as tb
+    m, n, k = 192, 320, 256
+    aq, bq, sa, sb = _int8_case(m, n, k, 52)
+    sa, sb = sa * 40.0, sb * 40.0          # push part of the results beyond +-127
+    c = torch.zeros(m, n, dtype=torch.int8, device="cuda")
+    tb.matmul_a8w8(aq.cuda(), bq.cuda().T.contiguous().T, sa.cuda(), sb.cuda(), c)
+    want = OG.ref_gemm_int8(aq, bq, torch.int8, a_scale=sa, b_scale=sb)
+    got = c.cpu()
+    assert int((want == 127).sum()) > 0 and int((want == -128).sum()) > 0 and int((want.abs() < 100).sum()) > 0
+    # the fp32 products acc*(sa*sb) of kernel and oracle agree to the last bit or the one before;
+    # truncation can turn that into a difference of 1 right at an integer
+    diff = (got.to(torch.int32) - want.to(torch.int32)).abs()
+    assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) < 1e-3
+
+
 # ---- MXFP4 --------------------------------------------------------------------------------------
 def _fp4_case(m, n, k, seed):
     rng = np.random.default_rng(seed)

@@ -12,14 +12,14 @@ from oracle import gemm as OG
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float16: 1e-3, torch.bfloat16: 1e-3, torch.float32: 1e-5, torch.float8_e4m3fn: 1e-2}
+TOL = {torch.float16: 1e-3, torch.bfloat16: 1e-3, torch.float32: 1e-5, torch.float8_e4m3fn: 1e-2, torch.int8: 1e-3}
 
 
 def _cases(n, seed):
     rng = random.Random(seed)
     out = []
     for i in range(n):
-        dtype = rng.choice([torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn])
+        dtype = rng.choice([torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn, torch.int8])
         big = rng.random() < 0.3
         m = rng.randint(1, 1500 if big else 300)
         nn = rng.randint(1, 1500 if big else 300)
@@ -54,10 +54,13 @@ def test_random_case(case):
     dtype, m, n, k = case["dtype"], case["m"], case["n"], case["k"]
     g = torch.Generator().manual_seed(case["seed"])
     a32, b32 = torch.randn(m, k, generator=g) * 0.5, torch.randn(k, n, generator=g) * 0.5
-    quant = dtype == torch.float8_e4m3fn
+    quant = dtype in (torch.float8_e4m3fn, torch.int8)
     out_dtype = torch.bfloat16 if quant else dtype
     bias = (torch.randn(n, generator=g).to(out_dtype) if case["bias"] and not quant else None)
-    if quant:
+    if dtype == torch.int8:
+        a_cpu, sa = OG.quantize_per_channel_int8(a32, axis=1)
+        b_cpu, sb = OG.quantize_per_channel_int8(b32, axis=0)
+    elif quant:
         a_cpu, sa = OG.quantize_per_channel_fp8(a32, axis=1)
         b_cpu, sb = OG.quantize_per_channel_fp8(b32, axis=0)
     else:

@@ -30,18 +30,20 @@ FIELDNAMES = ["m", "n", "k", "mnk", "macro_tile", "bytes", "flops", "tritonblas_
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "float16": torch.float16, "fp16": torch.float16,
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float8_e4m3fn": torch.float8_e4m3fn,
-           "fp8": torch.float8_e4m3fn, "fp4": "fp4"}
+           "fp8": torch.float8_e4m3fn, "int8": torch.int8, "fp4": "fp4"}
 
 
 def str_to_dtype(name):
     key = str(name).replace("torch.", "").lower()
     if key not in _DTYPES:
-        raise ValueError(f"unsupported dtype {name!r}; this library runs float32, float16, bfloat16, float8_e4m3fn and fp4 inputs")
+        raise ValueError(f"unsupported dtype {name!r}; this library runs float32, float16, bfloat16, float8_e4m3fn, int8 and fp4 inputs")
     return _DTYPES[key]
 
 
 def _tolerances(in_dtype, out_dtype, quantized):
     if quantized:
+        if out_dtype == torch.int8:
+            return (2.0, 0.2)
         return (0.02, 1e-2) if out_dtype == torch.bfloat16 else (0.1, 0.05)
     return (0.5, 0.05)
 
@@ -70,7 +72,11 @@ def _make_case(m, n, k, in_dtype, out_dtype, transA, transB, init_type, enable_s
     if inp.scaleA is not None:
         launch = lambda: tb.matmul_a8w8_lt(inp.A, inp.B, inp.scaleA, inp.scaleB, inp.C, sel, cfg, enable_streamk,
                                            work_stealing=work_stealing)
-        ref = lambda: ((inp.A.float() @ inp.B.float()) * (inp.scaleA[:, None] * inp.scaleB[None, :])).to(out_dtype)
+        def ref():
+            acc = (inp.A.float() @ inp.B.float()) * (inp.scaleA[:, None] * inp.scaleB[None, :])
+            if out_dtype == torch.int8:   # (reference benchmarks/tritonblas_matmul.py:72-74)
+                acc = torch.clamp(acc, -127.0, 127.0)
+            return acc.to(out_dtype)
     else:
         launch = lambda: tb.matmul_lt(inp.A, inp.B, inp.C, sel, cfg, enable_streamk, work_stealing=work_stealing)
         ref = lambda: torch.matmul(inp.A, inp.B).to(out_dtype)

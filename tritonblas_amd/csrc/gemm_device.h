@@ -18,7 +18,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
-enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4 };
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4, DT_I8 = 5 };
 enum : int { MODE_STATIC = 0, MODE_WS = 1, MODE_SK = 2, MODE_GROUPED = 3 };
 enum : int { WS_QUEUES = 0, WS_GLOBAL = 1, WS_HIERARCHICAL = 2 };   // how work-stealing workgroups find tiles
 enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
@@ -421,6 +421,9 @@ __device__ __forceinline__ v4f mma(typename Frag<T>::type x, typename Frag<T>::t
     c = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[1], yf[1], c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_16x16x4f32(xf[2], yf[2], c, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_16x16x4f32(xf[3], yf[3], c, 0, 0, 0);
+  } else if constexpr (T::DT == DT_I8) {
+    // exact int32 sums: the accumulator registers hold integers until the K loop ends
+    return __builtin_bit_cast(v4f, __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, __builtin_bit_cast(v4i, c), 0, 0, 0));
   } else if constexpr (T::DT == DT_FP8) {
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
   } else {
@@ -783,6 +786,16 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       __syncthreads();
     }
   }
+  if constexpr (T::DT == DT_I8) {
+    // int32 sums -> fp32 once per K range (exact below 2^24; Stream-K partials and the epilogue work in fp32)
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j) {
+        const v4i s32 = __builtin_bit_cast(v4i, acc[i][j]);
+        acc[i][j] = v4f{(float)s32.x, (float)s32.y, (float)s32.z, (float)s32.w};
+      }
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -797,7 +810,20 @@ __device__ __forceinline__ float load_as_f32(const uint8_t* p, int type) {
 
 template <int CT>
 __device__ __forceinline__ void store4(uint8_t* C, int64_t off_el, int64_t sn, v4f v, int nvalid, bool vec) {
-  if constexpr (CT == DT_F32) {
+  if constexpr (CT == DT_I8) {
+    // fp32 -> int8: toward zero, saturated to [-128, 127] (NaN -> 0)
+    uint32_t b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float t = __builtin_truncf(v[j]);
+      t = t != t ? 0.f : fminf(fmaxf(t, -128.f), 127.f);
+      b[j] = (uint32_t)(int)t & 0xFFu;
+    }
+    uint8_t* cp = C + off_el;
+    if (vec && nvalid >= 4) { *(uint32_t*)cp = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24); return; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (j < nvalid) cp[j * sn] = (uint8_t)b[j];
+  } else if constexpr (CT == DT_F32) {
     float* cp = (float*)C + off_el;
     if (vec && nvalid >= 4) { *(v4f*)cp = v; return; }
 #pragma unroll
@@ -970,6 +996,9 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc,
     else if (p.c_type == DT_F16) epilogue_lines<T, DT_F16>(p, tc, acc, li, lds);
     else epilogue_lines<T, DT_F32>(p, tc, acc, li, lds);
     return;
+  }
+  if constexpr (T::DT == DT_I8) {
+    if (p.c_type == DT_I8) { epilogue_t<T, DT_I8>(p, tc, acc, li); return; }
   }
   if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);
   else if (p.c_type == DT_F16) epilogue_t<T, DT_F16>(p, tc, acc, li);

@@ -31,5 +31,7 @@ extern const Variant g_variants_fp4[];
 extern const int g_num_variants_fp4;
 extern const Variant g_variants_f32[];
 extern const int g_num_variants_f32;
+extern const Variant g_variants_i8[];
+extern const int g_num_variants_i8;
 
 }  // namespace tb

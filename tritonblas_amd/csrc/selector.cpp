@@ -12,7 +12,7 @@ namespace tb {
 static int type_bits(int t) {
   switch (t) {
     case TB_F16: case TB_BF16: return 16;
-    case TB_FP8_E4M3: return 8;
+    case TB_FP8_E4M3: case TB_I8: return 8;
     case TB_FP4_E2M1: return 4;
     case TB_F32: return 32;
   }
@@ -23,7 +23,7 @@ static int type_bits(int t) {
 static double mfma_flops_per_clk(int t) {
   switch (t) {
     case TB_F16: case TB_BF16: return 4096.0;
-    case TB_FP8_E4M3: return 8192.0;
+    case TB_FP8_E4M3: case TB_I8: return 8192.0;
     case TB_FP4_E2M1: return 16384.0;
     case TB_F32: return 256.0;
   }
@@ -82,7 +82,7 @@ static double family_efficiency(int dt, const TileInfo& v) {
   static const double h16[4] = {0.59, 0.50, 0.22, 0.12};
   static const double f4[4] = {0.45, 0.36, 0.22, 0.10};
   static const double f32[4] = {0.80, 0.75, 0.60, 0.30};   // the fp32 matrix pipe is slow enough to hide everything else
-  if (dt == TB_FP8_E4M3) return f8[cls];
+  if (dt == TB_FP8_E4M3 || dt == TB_I8) return f8[cls];
   if (dt == TB_FP4_E2M1) return f4[cls];
   if (dt == TB_F32) return f32[cls];
   return h16[cls];

@@ -72,6 +72,7 @@ void variant_table(int dt, const Variant** v, int* n) {
     case TB_FP8_E4M3: *v = g_variants_fp8; *n = g_num_variants_fp8; break;
     case TB_FP4_E2M1: *v = g_variants_fp4; *n = g_num_variants_fp4; break;
     case TB_F32: *v = g_variants_f32; *n = g_num_variants_f32; break;
+    case TB_I8: *v = g_variants_i8; *n = g_num_variants_i8; break;
     default: *v = nullptr; *n = 0;
   }
 }
@@ -119,7 +120,7 @@ int default_panel_n(int grid, int chunk, int group_m) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : (dt == TB_F32 ? 4 : 1); }
-int c_bytes(int t) { return t == TB_F32 ? 4 : 2; }
+int c_bytes(int t) { return t == TB_F32 ? 4 : (t == TB_I8 ? 1 : 2); }
 
 // Everything the launch path needs, independent of which public descriptor it came from.
 struct Job {
@@ -164,7 +165,7 @@ int kernel_occupancy(const Variant* v, const void* kernel) {
 int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
   if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
-  if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32) return TB_ERR_BAD_DTYPE;
+  if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8)) return TB_ERR_BAD_DTYPE;
   const int usz = unit_bytes(j.dt);
   const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
   if (j.K % epu) return TB_ERR_BAD_SHAPE;
@@ -239,7 +240,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.a_vec = p.b_vec = v->fast;
   const int cb = c_bytes(j.c_type);
   p.c_vec = (j.c_sn == 1 && (j.c_sm % 4 == 0 || j.M == 1) && ((uintptr_t)j.C % (4 * cb)) == 0) ? 1 : 0;
-  p.c_line = (j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
+  p.c_line = (j.c_type != TB_I8 && j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
   { const char* e = getenv("TB_NO_CLINE"); if (e && atoi(e)) p.c_line = 0; }
   if (j.dt == TB_FP4_E2M1) {
     const int ksub = v->bk / 128;
@@ -360,7 +361,7 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
   if (d->a_type != d->b_type) return TB_ERR_BAD_DTYPE;
-  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_F32) return TB_ERR_BAD_DTYPE;
+  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_F32 && d->a_type != TB_I8) return TB_ERR_BAD_DTYPE;
   if ((d->a_scale == nullptr) != (d->b_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
   if (d->bias && d->bias_type != TB_F16 && d->bias_type != TB_BF16 && d->bias_type != TB_F32) return TB_ERR_BAD_DTYPE;
   j->dt = d->a_type; j->c_type = d->c_type; j->bias_type = d->bias_type;

@@ -19,14 +19,18 @@ def get_fp8_dtypes():
 def quantize_tensor_per_channel(tensor: torch.Tensor, target_dtype: torch.dtype, axis: int, *,
                                 min_scale: float = 1e-8) -> Tuple[torch.Tensor, torch.Tensor]:
     """amax along ``axis`` -> scale = amax / dtype_max -> q = (x * (1/scale)).to(dtype); returns
-    (q, scale squeezed along axis, fp32).  Reference utils.py:340-377."""
-    if target_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
+    (q, scale squeezed along axis, fp32).  int8: dtype_max = 127, q rounded to nearest and clamped
+    to [-127, 127] first.  Reference utils.py:340-377."""
+    if target_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2, torch.int8):
         raise ValueError(f"Unsupported quantized dtype: {target_dtype}")
     base = tensor.to(torch.float32)
     max_abs = torch.clamp(base.abs().amax(dim=axis, keepdim=True), min=min_scale)
-    scale = max_abs / torch.finfo(target_dtype).max
-    q = (base * (1.0 / scale)).to(target_dtype)
-    return q, scale.squeeze(axis).to(torch.float32)
+    dtype_max = 127.0 if target_dtype == torch.int8 else torch.finfo(target_dtype).max
+    scale = max_abs / dtype_max
+    q = base * (1.0 / scale)
+    if target_dtype == torch.int8:
+        q = torch.round(q).clamp_(-dtype_max, dtype_max)
+    return q.to(target_dtype), scale.squeeze(axis).to(torch.float32)
 
 
 _E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]
@@ -129,7 +133,7 @@ def generate_matmul_inputs(m, n, k, in_dtype, out_dtype=torch.float16, transA="T
         A, scaleA = dynamic_mxfp4_quant(A.contiguous())
         Bq, scaleB = dynamic_mxfp4_quant(B.T.contiguous())
         B = Bq.T
-    elif in_dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+    elif in_dtype in (torch.float8_e4m3fn, torch.float8_e5m2, torch.int8):
         A, scaleA = quantize_tensor_per_channel(A, in_dtype, axis=1)
         B, scaleB = quantize_tensor_per_channel(B, in_dtype, axis=0)
     else:
