@@ -194,7 +194,7 @@ def main():
         sec["fp32_gemm_8192x8192x8192_TN"] = {"ms": round(f32ms, 4), "TFLOP/s": round(tf3, 1),
                                               "frac_mfma_peak": round(tf3 / PEAK_TFLOPS["fp32"], 4)}
         del a3, b3, c3
-        # FP8 decode: the library routes M <= 64 to its streaming kernel (weight read once, split-K inside the workgroup)
+        # FP8 decode: for M <= 64 the library compares the model times of its streaming kernel and of the Stream-K tile kernel
         Md, Nd, Kd = 32, 8192, 28672
         aqd, wqd, sad, swd = fp8_inputs(Md, Nd, Kd, dev, 22)
         cd = torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev)
@@ -204,8 +204,9 @@ def main():
         dbytes = Md * Kd + Nd * Kd + Md * Nd * 2 + (Md + Nd) * 4
         sec["fp8_decode_32x8192x28672"] = {"ms": round(dms, 4), "GB/s": round(dbytes / dms / 1e6, 1),
                                            "frac_hbm_peak": round(dbytes / dms / 1e6 / PEAK_HBM_GBPS, 4),
-                                           "kernel": "streaming skinny-M kernel (enable_streamk=True call; Stream-K tiles are the "
-                                                     "fallback for shapes it does not cover)"}
+                                           "kernel": f"enable_streamk=True call; the library picks between the Stream-K tile kernel "
+                                                     f"(selector: {seld.block_m}x{seld.block_n}x{seld.block_k} tiles, grid {seld.sk_grid}) "
+                                                     f"and its streaming small-M kernel by model time"}
         del aqd, wqd, cd
         # grouped MoE FP8
         E, Ng, Kg, T = 8, 14336, 4096, 4096

@@ -316,11 +316,10 @@ def test_streamk_workspace_reuse_with_new_data(m, n, k, grid):
 @pytest.mark.parametrize("kernel", ["streaming", "streamk"])
 def test_decode_shape_small(kernel, monkeypatch):
     """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly:
-    through the streaming skinny-M kernel the library picks, and through the tile kernel's Stream-K
-    fixup (TB_NO_SKINNY switches the streaming kernel off)."""
+    through the streaming skinny-M kernel and through the tile kernel's Stream-K fixup (the library
+    picks between them by model time; TB_SKINNY / TB_NO_SKINNY force the choice)."""
     import tritonblas_amd as tb
-    if kernel == "streamk":
-        monkeypatch.setenv("TB_NO_SKINNY", "1")
+    monkeypatch.setenv("TB_NO_SKINNY" if kernel == "streamk" else "TB_SKINNY", "1")
     m, n, k = 32, 1024, 7168
     aq, bq, sa, sb = _a8w8_case(m, n, k, seed=21)
     a, b = aq.cuda(), bq.T.contiguous().cuda().T
@@ -336,11 +335,15 @@ def test_decode_shape_small(kernel, monkeypatch):
 @pytest.mark.parametrize("m,n,k", [(m, 1040, 2304) for m in (1, 5, 16, 17, 32, 33, 64)] +
                          [(m, 24576 + 40, 256) for m in (7, 32, 64)])   # wide N: 64-column workgroups
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
-def test_skinny_rows(m, n, k, dtype):
+@pytest.mark.parametrize("forced", [True, False])
+def test_skinny_rows(m, n, k, dtype, forced, monkeypatch):
     """Every row-block count of the streaming kernel and both column widths of its workgroups, ragged N,
-    bias, all three element types."""
+    bias, all three element types; once forced onto the streaming kernel, once with the library's own
+    choice between it and the tile kernels."""
     import tritonblas_amd as tb
-    _say(f"skinny {m}x{n}x{k} {dtype}")
+    if forced:
+        monkeypatch.setenv("TB_SKINNY", "1")
+    _say(f"skinny {m}x{n}x{k} {dtype} forced={forced}")
     if dtype == torch.float8_e4m3fn:
         aq, bq, sa, sb = _a8w8_case(m, n, k, seed=31)
         c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")

@@ -88,14 +88,18 @@ static double family_efficiency(int dt, const TileInfo& v) {
   return h16[cls];
 }
 
-// Stream-K launch grid for `total` tiles of `k_iters` K steps on `slots` co-resident workgroups.
-//   * fewer tiles than slots: every tile is cut into the same number s of K segments (grid = total * s),
+// Stream-K launch grid for `total` tiles of `k_iters` K steps on `slots` co-resident workgroups of `n_cu` CUs.
+//   * at least one whole tile per CU, but fewer tiles than slots: one workgroup per tile, nothing is
+//     split -- every CU is busy, and cutting tiles only to raise the occupancy costs more in partial-tile
+//     traffic than it gains (measured: 64x28672x8192 fp8, 448 tiles of 64x64: 38 us whole, 60 us in halves);
+//   * fewer tiles than CUs: every tile is cut into the same number s of K segments (grid = total * s),
 //     as many as fit the slots but never shorter than 16 K steps -- below that the fixup (one partial
 //     tile written, polled for and added per extra segment) costs more than the split saves;
-//   * otherwise every slot takes part: whole tiles first, the last total % slots tiles are shared.
-int streamk_grid(int64_t total, int64_t k_iters, int slots) {
+//   * tiles >= slots: every slot takes part: whole tiles first, the last total % slots tiles are shared.
+int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu) {
   if (total <= 0 || slots <= 0) return 1;
   if (total >= slots) return slots;
+  if (total >= n_cu) return (int)total;
   int64_t s = std::max<int64_t>(1, slots / total);
   s = std::min<int64_t>(s, std::max<int64_t>(1, k_iters / 16));
   return (int)(total * s);
@@ -120,10 +124,12 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   double us;
   if (streamk) {
     // one extra K segment of a tile costs its partial tile written through, polled for and added by the
-    // owner, one after the other: ~2 us + the fp32 tile at ~50 GB/s
-    const double fix_us = 2.0 + area * 4.0 / 50e3;
+    // owner, one after the other, plus the segment's own start-up: ~4 us + the fp32 tile at ~25 GB/s
+    // (fitted: 256x8192x8192 fp8 in four segments of 128x128 tiles 45 us, 128x4096x14336 bf16 in eight
+    // segments of 64x64 tiles 67 us)
+    const double fix_us = 4.0 + area * 4.0 / 25e3;
     const int slots = hw.n_cu * occ;
-    const int grid = streamk_grid(tiles, k_iters, slots);
+    const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu);
     const double w = (double)cdiv(grid, hw.n_cu);                 // workgroups sharing the busiest CU
     const double t_step = std::max(w * t_thru, t_lat);
     const int64_t dp_rounds = tiles / grid, tail = tiles % grid;
@@ -151,6 +157,22 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   const double hbm = std::min(hw.hbm_gbps * 0.65, busy_cus * 45.0);
   *mem_us = (a_bytes + b_bytes + c_out) / (hbm * 1e9) * 1e6;
   return std::max(*comp_us, *mem_us) + 3.0;
+}
+
+double estimate_tile_us(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk) {
+  double c, m;
+  return score(pr, hw, v, streamk, &c, &m);
+}
+
+// The streaming kernel for a handful of rows: every workgroup owns 64 columns of the weight, reads them
+// once from HBM (measured ~4.6 TB/s over the whole grid) and re-reads all of A from L2 (~17 TB/s over
+// the grid); ~9 us of launch, split-K reduction and store on top.
+double estimate_streaming_us(const tb_problem& pr, const tb_hw& hw) {
+  const double esz = type_bits(pr.a_type) / 8.0;
+  const double b_bytes = (double)pr.n * pr.k * esz;
+  const double a_reread = std::ceil(pr.n / 64.0) * (double)pr.m * pr.k * esz;
+  const double hbm = hw.hbm_gbps * 0.575 * 1e3, l2 = hw.hbm_gbps * 2.125 * 1e3;   // bytes per us
+  return 9.0 + b_bytes / hbm + a_reread / l2;
 }
 
 int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out) {
@@ -191,7 +213,7 @@ int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, in
   out->num_stages = v.stages;
   out->lds_bytes = v.lds_bytes;
   out->counters_per_xcd = ws_counters_per_xcd(total);
-  out->sk_grid = streamk_grid(total, cdiv(pr.k, v.bk), hw.n_cu * out->occupancy);
+  out->sk_grid = streamk_grid(total, cdiv(pr.k, v.bk), hw.n_cu * out->occupancy, hw.n_cu);
   out->est_compute_us = best_c; out->est_memory_us = best_m; out->est_total_us = best_t;
   return TB_OK;
 }

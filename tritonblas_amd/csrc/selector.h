@@ -10,11 +10,14 @@ struct TileInfo {
 };
 
 void default_hw(tb_hw* hw);
-int streamk_grid(int64_t total_tiles, int64_t k_iters, int slots);
+int streamk_grid(int64_t total_tiles, int64_t k_iters, int slots, int n_cu);
 int ws_counters_per_xcd(int64_t total_tiles);
 // (tiles per XCD-local queue, tiles in the shared pool) of the hierarchical work-stealing mode
 void hierarchical_split(int64_t total_tiles, int hw_cus, int num_xcds, int64_t* local_per_xcd, int64_t* global_tiles);
 int variant_occupancy(const TileInfo& v, const tb_hw& hw);
 int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out);
+// model time (us) of one tile variant on a problem, and of the streaming small-M kernel
+double estimate_tile_us(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk);
+double estimate_streaming_us(const tb_problem& pr, const tb_hw& hw);
 
 }  // namespace tb

@@ -263,10 +263,22 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
 
   const void* kern = (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) ? v->kernel_sk : v->kernel;
   {
-    // a handful of rows against a K-major weight: the streaming kernel reads B once at HBM rate
+    // a handful of rows against a K-major weight: the streaming kernel (no tiles, no workspace) when
+    // the model expects it to beat the tile kernel of the requested schedule.  TB_NO_SKINNY=1 / TB_SKINNY=1
+    // force the choice (tuning and tests).
     const char* e = getenv("TB_NO_SKINNY");
+    const char* f = getenv("TB_SKINNY");
     plan->skinny = j.num_groups == 0 && skinny_supported(j.dt, j.M) && alay == LAY_K && blay == LAY_K &&
                    KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !(e && atoi(e));
+    if (plan->skinny && !(f && atoi(f))) {
+      tb_problem pr;
+      std::memset(&pr, 0, sizeof(pr));
+      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+      pr.a_k_contiguous = pr.b_k_contiguous = 1;
+      const bool sk = j.schedule == TB_SCHED_STREAMK;
+      const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, v->minb, v->fast, v->stages};
+      plan->skinny = estimate_streaming_us(pr, hw) < estimate_tile_us(pr, hw, ti, sk);
+    }
     if (plan->skinny) { plan->v = v; plan->grid = 1; plan->ws_need = 0; return TB_OK; }
   }
   const int occ = need_device ? kernel_occupancy(v, kern) : std::max(1, std::min(v->minb, hw.lds_bytes / v->lds_bytes));
@@ -307,7 +319,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     plan->ws_need = plan->ws_counters_off + ((size_t)p.num_xcds * p.counters_per_xcd + 1) * COUNTER_STRIDE * 4;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
-    int64_t g = j.grid > 0 ? j.grid : streamk_grid(total, p.k_iters, resident);
+    int64_t g = j.grid > 0 ? j.grid : streamk_grid(total, p.k_iters, resident, hw.n_cu);
     if (g > resident) return TB_ERR_BAD_SCHEDULE;  // owners spin on later workgroups: all must be resident
     grid = (int)g;
     p.sk_tiles = (int32_t)(total % grid);
