@@ -77,6 +77,38 @@ def test_every_16bit_tile_variant(m, n, k, dtype, tile):
         _check(c.cpu(), want, dtype, TOL_16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("stages", [3, 4])
+@pytest.mark.parametrize("m,n,k", [(128, 512, 4096), (300, 200, 2304), (64, 64, 128), (512, 1024, 640)])
+def test_deep_pipeline_variants_of_the_small_tile(dtype, stages, m, n, k, monkeypatch):
+    """The 64x64 tile exists with 2, 3 and 4 copy stages; the library takes a deeper one while all tiles
+    are resident at once.  Here every depth is forced (TB_WAVES = waves_m, waves_n, stages), K both
+    shorter and longer than the pipeline, ragged edges, Stream-K on top."""
+    import tritonblas_amd as tb
+    monkeypatch.setenv("TB_WAVES", f"22{stages}")
+    monkeypatch.setenv("TB_NO_SKINNY", "1")
+    _say(f"deep pipeline {dtype} stages={stages} {m}x{n}x{k}")
+    quant = dtype == torch.float8_e4m3fn
+    if quant:
+        aq, bq, sa, sb = _a8w8_case(m, n, k, seed=61)
+        a, b = aq.cuda(), bq.T.contiguous().cuda().T
+        want, out_dtype, tol = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb), torch.bfloat16, TOL_Q
+    else:
+        a_cpu, b_cpu = _rand((m, k), dtype, 62, 0.5), _rand((k, n), dtype, 63, 0.5)
+        a, b = a_cpu.cuda(), b_cpu.T.contiguous().cuda().T
+        want, out_dtype, tol = OG.ref_gemm(a_cpu, b_cpu, torch.float32), dtype, TOL_16
+    for sk in (False, True):
+        sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, out_dtype, a.device, streamk=sk)
+        sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 64, 64, (128 if quant else 64)
+        cfg = tb.matmul_preamble(sel)
+        c = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        if quant:
+            tb.matmul_a8w8_lt(a, b, sa.cuda(), sb.cuda(), c, sel, cfg, enable_streamk=sk)
+        else:
+            tb.matmul_lt(a, b, c, sel, cfg, enable_streamk=sk)
+        _check(c.cpu(), want, out_dtype, tol)
+
+
 def test_config1_fp16_1024():
     import tritonblas_amd as tb
     a_cpu, b_cpu = OI.c1_fp16()

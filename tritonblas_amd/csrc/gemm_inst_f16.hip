@@ -14,6 +14,10 @@ const Variant g_variants_f16[] = {
     TB_LAYOUTS(256, 256, 2, 4, 1),
     TB_LAYOUTS(128, 128, 2, 2, 2),
     TB_LAYOUTS(64, 64, 2, 2, 4),
+    // deeper copy pipelines of the small tile for problems with few tiles per CU (each K step then
+    // waits less for its copy; fewer workgroups fit a CU)
+    make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 3, true, 3>>(),
+    make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, true, 4>>(),
     make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),
 };
 const int g_num_variants_f16 = sizeof(g_variants_f16) / sizeof(Variant);

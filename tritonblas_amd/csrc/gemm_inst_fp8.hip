@@ -9,6 +9,10 @@ const Variant g_variants_fp8[] = {
     make_variant<Tile<DT_FP8, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),
     make_variant<Tile<DT_FP8, 32, 128, 256, 1, 4, LAY_K, LAY_K, 1, true, 3>>(),
+    // deeper copy pipelines of the small tile for problems with few tiles per CU (each K step then
+    // waits less for its copy; fewer workgroups fit a CU)
+    make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 3, true, 3>>(),
+    make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, true, 4>>(),
     make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),
 };
 const int g_num_variants_fp8 = sizeof(g_variants_fp8) / sizeof(Variant);

@@ -90,7 +90,13 @@ std::vector<TileInfo> tile_infos(int dt) {
   return out;
 }
 
-const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast) {
+// Variants may share a tile shape and differ in the depth of the copy pipeline.  A deeper pipeline hides
+// more of the copy latency of every K step but lets fewer workgroups share a CU, so it only pays while
+// all tiles are resident at once: the deepest variant that still holds `total_tiles` on the device is
+// taken (measured, 64x64 bf16 tiles: 128x4096x4096 32 -> 22 us, 64x8192x8192 60 -> 39 us with four
+// stages; 2048^3 30 -> 35 us, which the rule avoids).
+const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast, int64_t total_tiles = 0,
+                            const tb_hw* hw = nullptr) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
   // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
@@ -101,10 +107,15 @@ const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, 
       if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
           (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want))
         return &v[i];
-  for (int i = 0; i < n; ++i)
-    if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk)))
-      return &v[i];
-  return nullptr;
+  const Variant* best = nullptr;
+  for (int i = 0; i < n; ++i) {
+    if (!(v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk))))
+      continue;
+    if (!best) { best = &v[i]; if (!hw || total_tiles <= 0 || !fast) return best; continue; }   // (listed first: the default depth)
+    const int occ = std::max(1, std::min(v[i].minb, hw->lds_bytes / std::max(1, v[i].lds_bytes)));
+    if (v[i].stages > best->stages && total_tiles <= (int64_t)hw->n_cu * occ) best = &v[i];
+  }
+  return best;
 }
 
 // Width (in tiles) of the column panels of the tile order.  One pass of the grid over the tile list
@@ -213,7 +224,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       fast = false;
   }
   if (fast) {
-    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1);
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, j.num_groups > 0 ? 0 : ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn), &hw);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
