@@ -118,7 +118,15 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
 
   const double ideal_step_us = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type) / clk * 1e6;
   const double t_thru = ideal_step_us / family_efficiency(pr.a_type, v);   // CU time per tile K step, saturated
-  const double t_lat = 0.30 + (v.bm + v.bn) * (v.bk * esz) / 1.0e5;          // floor per K step of one workgroup: round trip + its own copy at ~100 GB/s
+  double t_lat = 0.30 + (v.bm + v.bn) * (v.bk * esz) / 1.0e5;                // floor per K step of one workgroup: round trip + its own copy at ~100 GB/s
+  // the 64x64 tile of the 8- and 16-bit float types runs with four (three) copy stages while no more
+  // than two (three) tiles per CU exist, which hides that much more of the round trip (measured x0.67 / x0.85)
+  if (v.bm == 64 && v.bn == 64 && pr.num_groups == 0 &&
+      (pr.a_type == TB_F16 || pr.a_type == TB_BF16 || pr.a_type == TB_FP8_E4M3)) {
+    const int64_t whole = cdiv(pr.m, v.bm) * cdiv(pr.n, v.bn);
+    if (whole <= 2 * (int64_t)hw.n_cu) t_lat *= 0.67;
+    else if (whole <= 3 * (int64_t)hw.n_cu) t_lat *= 0.85;
+  }
   const double t_tile = area >= 256 * 256 ? 12.0 : (area >= 128 * 128 ? 4.0 : 3.0);
 
   double us;

@@ -224,7 +224,12 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       fast = false;
   }
   if (fast) {
-    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, j.num_groups > 0 ? 0 : ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn), &hw);
+    // workgroups that have to be resident at once for a deeper-pipeline variant to be the better one:
+    // all tiles, and for Stream-K the whole grid (the owners wait for the other segments' workgroups)
+    int64_t at_once = ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn);
+    if (j.schedule == TB_SCHED_STREAMK) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
+    if (j.num_groups > 0) at_once = 0;
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
