@@ -60,7 +60,7 @@ def test_matmul_16bit(m, n, k, dtype, transA, transB):
 
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (512, 768, 320), (300, 200, 192), (257, 129, 64)])
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("tile", [(256, 256, 64), (128, 128, 64), (64, 64, 64)])
+@pytest.mark.parametrize("tile", [(256, 256, 64), (128, 128, 64), (64, 64, 64), (32, 128, 128)])
 def test_every_16bit_tile_variant(m, n, k, dtype, tile):
     """Forces each built tile through matmul_lt (the selector would otherwise pick one)."""
     import tritonblas_amd as tb

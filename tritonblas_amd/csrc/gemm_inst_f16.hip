@@ -18,6 +18,11 @@ const Variant g_variants_f16[] = {
     // waits less for its copy; fewer workgroups fit a CU)
     make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 3, true, 3>>(),
     make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, true, 4>>(),
+    // a handful of rows against a long K: short, wide, deep tile with three copy stages
+    make_variant<Tile<DT_F16, 32, 128, 256, 1, 4, LAY_K, LAY_K, 1, true, 3>>(),
+    make_variant<Tile<DT_F16, 32, 128, 256, 1, 4, LAY_K, LAY_M, 1, true, 2>>(),
+    make_variant<Tile<DT_F16, 32, 128, 256, 1, 4, LAY_M, LAY_K, 1, true, 2>>(),
+    make_variant<Tile<DT_F16, 32, 128, 256, 1, 4, LAY_M, LAY_M, 1, true, 2>>(),
     make_variant<Tile<DT_F16, 64, 64, 128, 2, 2, LAY_K, LAY_K, 2, false, 2>>(),
 };
 const int g_num_variants_f16 = sizeof(g_variants_f16) / sizeof(Variant);
