@@ -14,11 +14,23 @@ from .config import MatmulConfig, matmul_preamble
 from .origami import OrigamiMatmulSelector
 
 
+_SELECTOR_CACHE = {}
+_SELECTOR_CACHE_MAX = 4096
+
+
 def _make_matmul_selector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=0, streamk=False,
                           num_stages: int = 2):
-    """Reference matmul.py:42-66."""
-    return OrigamiMatmulSelector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=mx_block_size,
-                                 streamk=streamk, num_stages=num_stages)
+    """Reference matmul.py:42-66, which scores the tiles again on every call; here a selector is a pure
+    function of its arguments and is kept (the entry points that build their own selector call this)."""
+    key = (M, N, K, a_dtype, b_dtype, c_dtype, str(device), mx_block_size, bool(streamk), num_stages)
+    sel = _SELECTOR_CACHE.get(key)
+    if sel is None:
+        if len(_SELECTOR_CACHE) >= _SELECTOR_CACHE_MAX:
+            _SELECTOR_CACHE.clear()
+        sel = OrigamiMatmulSelector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=mx_block_size,
+                                    streamk=streamk, num_stages=num_stages)
+        _SELECTOR_CACHE[key] = sel
+    return sel
 
 
 def _ptr(t: Optional[torch.Tensor]):
