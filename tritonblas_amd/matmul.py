@@ -33,6 +33,24 @@ def _make_matmul_selector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_s
     return sel
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev):
+    """Context that makes ``dev`` the current device for a launch; free when it already is."""
+    if dev.index is None or torch.cuda.current_device() == dev.index:
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
@@ -115,7 +133,7 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
             ws = config.ensure(need)
             d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
             d.epoch = config.next_epoch()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
     return c
 
@@ -336,7 +354,7 @@ def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = 
         assert block_k % 64 == 0, "BLOCK_K must be multiple of 64 for FP4"
         d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
         d.group_m = group_size_m
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.load().tb_gemm_fp4(d, _lib.stream_handle(dev)), "tb_gemm_fp4")
     return c
 
@@ -368,6 +386,6 @@ def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int =
     d.group_offsets = _ptr(group_offsets)
     if block_m is not None:
         d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.load().tb_grouped_gemm_fp8(d, _lib.stream_handle(dev)), "tb_grouped_gemm_fp8")
     return c
