@@ -92,21 +92,40 @@ static double family_efficiency(int dt, const TileInfo& v) {
 //   * at least one whole tile per CU, but fewer tiles than slots: one workgroup per tile, nothing is
 //     split -- every CU is busy, and cutting tiles only to raise the occupancy costs more in partial-tile
 //     traffic than it gains (measured: 64x28672x8192 fp8, 448 tiles of 64x64: 38 us whole, 60 us in halves);
-//   * fewer tiles than CUs: every tile is cut into the same number s of K segments (grid = total * s),
-//     as many as fit the slots but never shorter than 16 K steps -- below that the fixup (one partial
-//     tile written, polled for and added per extra segment) costs more than the split saves;
-//   * tiles >= slots: every slot takes part: whole tiles first, the last total % slots tiles are shared.
-int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu) {
+//   * fewer tiles than CUs: every tile is cut into the same number s of K segments (grid = total * s).
+//     s is a power of two (segment counts that do not divide the K steps evenly were up to 2x slower:
+//     32x4096x14336 bf16, 112 steps: s = 4 and 8 28 us, s = 5..7 31..53 us), at most what fits the slots,
+//     never leaving fewer than 8 K steps per segment, and the one that minimises
+//     steps_per_segment * step_us + (s - 1) * fix_us -- the owner adds the other segments' partial tiles
+//     one after the other;
+//   * tiles >= slots: every slot takes part: whole tiles first, the last total % slots tiles are shared --
+//     unless another round of whole tiles is expected to be as fast (large tiles have expensive partial
+//     tiles: 2048x14336x4096 bf16, 448 tiles of 256x256 on 256 slots: 209 us in two rounds, 253 us with a
+//     shared tail); the return value `total` means "whole tiles only".
+int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us) {
   if (total <= 0 || slots <= 0) return 1;
-  if (total >= slots) return slots;
+  if (total >= slots) {
+    const int64_t tail = total % slots;
+    if (tail == 0) return slots;
+    const double shared = std::ceil((double)tail * k_iters / slots) * step_us + (std::ceil((double)slots / tail) - 1.0) * fix_us;
+    const double whole = (double)k_iters * step_us;
+    return shared < whole ? slots : (int)std::min<int64_t>(total, INT32_MAX);
+  }
   if (total >= n_cu) return (int)total;
-  int64_t s = std::max<int64_t>(1, slots / total);
-  s = std::min<int64_t>(s, std::max<int64_t>(1, k_iters / 16));
-  return (int)(total * s);
+  const int64_t smax = std::max<int64_t>(1, slots / total);
+  int64_t best_s = 1;
+  double best = 0;
+  for (int64_t s2 = 1; s2 <= smax && (s2 == 1 || k_iters / s2 >= 8); s2 *= 2) {
+    // workgroups per CU grow with the split; beyond one per CU they share its matrix pipe
+    const double share = std::max(1.0, (double)(total * s2) / n_cu);
+    const double cost = std::ceil((double)k_iters / s2) * step_us * std::sqrt(share) + (s2 - 1) * fix_us;
+    if (s2 == 1 || cost < best) { best = cost; best_s = s2; }
+  }
+  return (int)(total * best_s);
 }
 
 static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk, double* comp_us,
-                    double* mem_us) {
+                    double* mem_us, int* sk_grid_out = nullptr) {
   const double clk = hw.clock_khz * 1e3;
   const int bits = type_bits(pr.a_type);
   const double esz = bits / 8.0;
@@ -132,20 +151,25 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   double us;
   if (streamk) {
     // one extra K segment of a tile costs its partial tile written through, polled for and added by the
-    // owner, one after the other, plus the segment's own start-up: ~4 us + the fp32 tile at ~25 GB/s
-    // (fitted: 256x8192x8192 fp8 in four segments of 128x128 tiles 45 us, 128x4096x14336 bf16 in eight
-    // segments of 64x64 tiles 67 us)
-    const double fix_us = 4.0 + area * 4.0 / 25e3;
+    // owner, one after the other: ~1.5 us + the fp32 tile at ~10 GB/s (fitted on segment-count sweeps:
+    // 32x128 tiles ~3 us, 128x128 tiles ~8 us, 256x256 tiles ~30 us per extra segment)
+    const double fix_us = 1.5 + area * 4.0 / 10e3;
     const int slots = hw.n_cu * occ;
-    const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu);
-    const double w = (double)cdiv(grid, hw.n_cu);                 // workgroups sharing the busiest CU
+    const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu, std::max(t_thru, t_lat), fix_us);
+    if (sk_grid_out) *sk_grid_out = grid;
+    const int launched = (int)std::min<int64_t>(grid, slots);     // (grid == tiles > slots: whole tiles, resident grid loops)
+    const double w = (double)cdiv(launched, hw.n_cu);             // workgroups sharing the busiest CU
     const double t_step = std::max(w * t_thru, t_lat);
-    const int64_t dp_rounds = tiles / grid, tail = tiles % grid;
-    us = (double)dp_rounds * (k_iters * t_step + t_tile);
-    if (tail > 0) {
-      const double iters = std::ceil((double)tail * k_iters / grid);
-      const double segments = std::ceil((double)grid / tail);
-      us += iters * t_step + (segments - 1.0) * fix_us + t_tile;
+    if (grid >= tiles && tiles > slots) {
+      us = (double)cdiv(tiles, slots) * (k_iters * t_step + t_tile);
+    } else {
+      const int64_t dp_rounds = tiles / grid, tail = tiles % grid;
+      us = (double)dp_rounds * (k_iters * t_step + t_tile);
+      if (tail > 0) {
+        const double iters = std::ceil((double)tail * k_iters / grid);
+        const double segments = std::ceil((double)grid / tail);
+        us += iters * t_step + (segments - 1.0) * fix_us + t_tile;
+      }
     }
   } else {
     // the busiest CU works through c tiles, occ at a time
@@ -167,20 +191,28 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   return std::max(*comp_us, *mem_us) + 3.0;
 }
 
+int streamk_grid_for(const tb_problem& pr, const tb_hw& hw, const TileInfo& v) {
+  double c, m;
+  int grid = 1;
+  score(pr, hw, v, true, &c, &m, &grid);
+  return grid;
+}
+
 double estimate_tile_us(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bool streamk) {
   double c, m;
   return score(pr, hw, v, streamk, &c, &m);
 }
 
 // The streaming kernel for a handful of rows: every workgroup owns 64 columns of the weight, reads them
-// once from HBM (measured ~4.6 TB/s over the whole grid) and re-reads all of A from L2 (~17 TB/s over
-// the grid); ~9 us of launch, split-K reduction and store on top.
+// once from HBM (measured over the whole grid: ~4.6 TB/s with 8-bit operands, ~3.4 TB/s with 16-bit
+// ones) and re-reads all of A from L2 (~17 TB/s over the grid); ~13 us of launch, split-K reduction and
+// store on top.
 double estimate_streaming_us(const tb_problem& pr, const tb_hw& hw) {
   const double esz = type_bits(pr.a_type) / 8.0;
   const double b_bytes = (double)pr.n * pr.k * esz;
   const double a_reread = std::ceil(pr.n / 64.0) * (double)pr.m * pr.k * esz;
-  const double hbm = hw.hbm_gbps * 0.575 * 1e3, l2 = hw.hbm_gbps * 2.125 * 1e3;   // bytes per us
-  return 9.0 + b_bytes / hbm + a_reread / l2;
+  const double hbm = hw.hbm_gbps * (esz > 1.0 ? 0.425 : 0.575) * 1e3, l2 = hw.hbm_gbps * 2.125 * 1e3;   // bytes per us
+  return 13.0 + b_bytes / hbm + a_reread / l2;
 }
 
 int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, int ntiles, tb_selection* out) {
@@ -221,7 +253,7 @@ int select_tile(const tb_problem& pr, const tb_hw& hw, const TileInfo* tiles, in
   out->num_stages = v.stages;
   out->lds_bytes = v.lds_bytes;
   out->counters_per_xcd = ws_counters_per_xcd(total);
-  out->sk_grid = streamk_grid(total, cdiv(pr.k, v.bk), hw.n_cu * out->occupancy, hw.n_cu);
+  out->sk_grid = streamk_grid_for(pr, hw, v);
   out->est_compute_us = best_c; out->est_memory_us = best_m; out->est_total_us = best_t;
   return TB_OK;
 }

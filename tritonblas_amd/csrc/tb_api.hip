@@ -335,10 +335,22 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     plan->ws_need = plan->ws_counters_off + ((size_t)p.num_xcds * p.counters_per_xcd + 1) * COUNTER_STRIDE * 4;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
-    int64_t g = j.grid > 0 ? j.grid : streamk_grid(total, p.k_iters, resident, hw.n_cu);
+    int64_t g = j.grid;
+    if (g <= 0) {
+      tb_problem pr;
+      std::memset(&pr, 0, sizeof(pr));
+      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+      pr.a_k_contiguous = pr.b_k_contiguous = 1; pr.streamk = 1;
+      tb_hw hw_res = hw;   // (what the model may fill: the kernel's real occupancy)
+      const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, occ, v->fast, v->stages};
+      g = streamk_grid_for(pr, hw_res, ti);
+      if (g > resident) g = resident;
+    }
+    const bool whole_only = g == total;   // exactly one workgroup per tile (however many fit at once): nothing to share
+    if (whole_only) g = std::min<int64_t>(total, resident);
     if (g > resident) return TB_ERR_BAD_SCHEDULE;  // owners spin on later workgroups: all must be resident
     grid = (int)g;
-    p.sk_tiles = (int32_t)(total % grid);
+    p.sk_tiles = whole_only ? 0 : (int32_t)(total % grid);
     if (p.sk_tiles == 0) {
       // nothing to share: the same tiles on the whole-tile kernel (identical results, no workspace)
       p.mode = MODE_STATIC;
