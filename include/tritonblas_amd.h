@@ -129,7 +129,8 @@ typedef struct tb_gemm_desc {
   int32_t block_m, block_n, block_k;  /* tile variant, from tb_select; 0 = let the library select    */
   int32_t group_m, num_xcds;
   int32_t schedule;           /* TB_SCHED_*                                                         */
-  int32_t grid;               /* workgroups to launch; 0 = default (what is co-resident)            */
+  int32_t grid;               /* workgroups to launch; 0 = default (what is co-resident).  A Stream-K
+                                 grid beyond what is co-resident is replaced by the default          */
   int32_t counters_per_xcd;
   void* workspace;            /* tb_workspace_bytes() bytes, zero-initialised once by the caller     */
   size_t workspace_bytes;

@@ -462,6 +462,23 @@ def test_addmm_fp32(out_dtype):
     assert err <= (TOL_32 if out_dtype == torch.float32 else TOL_16), f"{err:.3e}"
 
 
+def test_streamk_grid_sized_for_another_tile():
+    """The selector sizes its Stream-K grid for the tile it picked; operands that need the gather kernel
+    run another tile with fewer co-resident workgroups.  The library then chooses the grid itself
+    instead of refusing the launch."""
+    import tritonblas_amd as tb
+    m, n, k = 1261, 670, 2688
+    a_cpu, b_cpu = _rand((m, k), torch.float32, 70, 0.5), _rand((k, n), torch.float32, 71, 0.5)
+    a, b = a_cpu.cuda(), b_cpu.cuda()          # B is N-contiguous: no LDS-direct fp32 kernel for it
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.float32, a.device, streamk=True)
+    cfg = tb.matmul_preamble(sel)
+    c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    tb.matmul_lt(a, b, c, sel, cfg, enable_streamk=True)
+    err = OG.rel_fro_error(c.cpu().double(), _ref64(a_cpu, b_cpu))
+    assert err <= TOL_32, f"{err:.3e}"
+    assert cfg.status() == 0
+
+
 # ---- int8 operands -------------------------------------------------------------------------------
 def _int8_case(m, n, k, seed):
     a = torch.randn(m, k, generator=torch.Generator().manual_seed(seed))

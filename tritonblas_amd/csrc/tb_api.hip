@@ -335,8 +335,11 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     plan->ws_need = plan->ws_counters_off + ((size_t)p.num_xcds * p.counters_per_xcd + 1) * COUNTER_STRIDE * 4;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
+    // (a requested grid that cannot be co-resident for the kernel that really runs -- the caller sized it
+    // for another tile, e.g. the operands turned out to need the gather kernel -- gives way to the
+    // library's own choice: owners wait for later workgroups, so all of them must be on the device)
     int64_t g = j.grid;
-    if (g <= 0) {
+    if (g <= 0 || g > resident) {
       tb_problem pr;
       std::memset(&pr, 0, sizeof(pr));
       pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
