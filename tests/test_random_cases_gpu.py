@@ -90,3 +90,77 @@ def test_random_case(case):
     assert torch.isfinite(got.float()).all(), "unwritten or non-finite outputs"
     err = OG.rel_fro_error(got.double(), want.float().to(out_dtype).double())
     assert err <= TOL[dtype], f"relative Frobenius error {err:.3e} > {TOL[dtype]}"
+
+
+def _fp4_cases(n, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        big = rng.random() < 0.3
+        out.append(dict(idx=i, m=rng.randint(1, 900 if big else 200), n=rng.randint(1, 900 if big else 200),
+                        k=32 * rng.choice([rng.randint(1, 40), 16 * rng.randint(1, 12), 16 * rng.randint(1, 12)]),
+                        tile=rng.choice([None, None, (256, 256, 256), (128, 128, 256), (128, 128, 128), (64, 64, 256)]),
+                        out=rng.choice([torch.bfloat16, torch.float16, torch.float32]), seed=rng.randint(0, 1 << 30)))
+    return out
+
+
+@pytest.mark.parametrize("case", _fp4_cases(max(8, int(os.environ.get("TB_RANDOM_CASES", "72")) // 3), 4242),
+                         ids=lambda c: f"{c['idx']}-{c['m']}x{c['n']}x{c['k']}-{c['tile']}")
+def test_random_fp4_case(case):
+    """MXFP4: random codes and random, widely varying E8M0 scales; K any multiple of 32 (multiples of 512
+    take the LDS-direct kernels, the rest the gather kernel), forced or selected tiles, three output types."""
+    import numpy as np
+    import tritonblas_amd as tb
+    print("random fp4 case", case, flush=True)
+    m, n, k = case["m"], case["n"], case["k"]
+    rng = np.random.default_rng(case["seed"])
+    xq = torch.from_numpy(rng.integers(0, 256, (m, k // 2), dtype=np.uint8))
+    wq = torch.from_numpy(rng.integers(0, 256, (n, k // 2), dtype=np.uint8))
+    hi = 129 if case["out"] == torch.float16 else 140      # (keep the sums inside the fp16 range)
+    xs = torch.from_numpy(rng.integers(110, hi, (m, k // 32), dtype=np.uint8))
+    ws = torch.from_numpy(rng.integers(110, hi, (n, k // 32), dtype=np.uint8))
+    c = torch.full((m, n), float("nan"), dtype=case["out"], device="cuda")
+    kw = {} if case["tile"] is None else dict(block_m=case["tile"][0], block_n=case["tile"][1], block_k=case["tile"][2])
+    tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda(), **kw)
+    want = OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True)
+    got = c.cpu()
+    assert torch.isfinite(got.float()).all()
+    err = OG.rel_fro_error(got.double(), want.to(case["out"]).double())
+    assert err <= (1e-5 if case["out"] == torch.float32 else 1e-3), f"relative Frobenius error {err:.3e}"
+
+
+def _grouped_cases(n, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        experts = rng.randint(1, 9)
+        counts = [rng.choice([0, 1, rng.randint(1, 70), rng.randint(100, 600), 256, 257]) for _ in range(experts)]
+        out.append(dict(idx=i, counts=counts, n=rng.choice([64, 200, 384, 1000]), k=rng.choice([128, 512, 1152]),
+                        seed=rng.randint(0, 1 << 30)))
+    return out
+
+
+@pytest.mark.parametrize("case", _grouped_cases(max(6, int(os.environ.get("TB_RANDOM_CASES", "72")) // 6), 777),
+                         ids=lambda c: f"{c['idx']}-{sum(c['counts'])}rows-{len(c['counts'])}experts-{c['n']}x{c['k']}")
+def test_random_grouped_case(case):
+    """Grouped FP8 GEMM over random per-expert row counts (empty experts, single rows, ragged blocks)."""
+    import numpy as np
+    import tritonblas_amd as tb
+    print("random grouped case", case, flush=True)
+    counts, n, k = case["counts"], case["n"], case["k"]
+    m, E = sum(counts), len(counts)
+    if m == 0:
+        pytest.skip("no rows at all")
+    offsets = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)
+    g = torch.Generator().manual_seed(case["seed"])
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(E, n, k, generator=g).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    wq, sw = OG.quantize_per_channel_fp8(w, axis=2)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda())
+    want = OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True)
+    got = c.cpu()
+    assert torch.isfinite(got.float()).all()
+    err = OG.rel_fro_error(got.double(), want.to(torch.bfloat16).double())
+    assert err <= 1e-2, f"relative Frobenius error {err:.3e}"
