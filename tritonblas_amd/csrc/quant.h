@@ -15,6 +15,10 @@ struct QuantParams {
   int64_t x_stride;       // elements
   int64_t codes_stride;   // bytes
   int64_t scales_stride;  // bytes
+  // item index -> (row, column) without a 64-bit division while the item count fits 31 bits:
+  // row = mulhi(item, div_magic) >> div_shift (div_shift < 0: one item per row)
+  uint32_t div_magic;
+  int32_t div_shift;
 };
 
 hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, hipStream_t stream);
