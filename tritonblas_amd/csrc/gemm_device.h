@@ -46,6 +46,8 @@ struct GemmParams {
   int32_t c_type, bias_type;
   int32_t a_vec, b_vec, c_vec;   // 16-byte vector access is legal for this operand (c_vec: 4-element rows)
   int32_t c_line;                // C rows are 16-byte aligned with unit column stride: full-line store path
+  int32_t c_nt;                  // C is larger than the L2s together: store it non-temporal so that it
+                                 // does not push operand strips out of them
   int32_t mx_vec;                // scale rows can be read KSUB bytes at a time
   int32_t mx_lds;                // scale rows are 16-byte aligned and K/32 is a multiple of 32: stage scales in LDS
   int32_t tiles_m, tiles_n, total_tiles, k_iters;
@@ -973,7 +975,8 @@ __device__ __forceinline__ void epilogue_lines(const GemmParams& p, const TileCt
       const v4i val = *(const v4i*)(stage + row * RS + ch * 16);
       uint8_t* gp = p.C + ((int64_t)m * p.c_sm + n) * CS;
       if (n + 16 / CS <= tc.n_lim) {
-        *(v4i*)gp = val;
+        if (p.c_nt) __builtin_nontemporal_store(val, (v4i*)gp);
+        else *(v4i*)gp = val;
       } else {
         const uint32_t w[4] = {(uint32_t)val.x, (uint32_t)val.y, (uint32_t)val.z, (uint32_t)val.w};
 #pragma unroll
