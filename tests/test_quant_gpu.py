@@ -41,6 +41,20 @@ def test_random(shape, dtype, hadamard):
 
 
 @pytest.mark.parametrize("hadamard", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 32), (3, 64), (257, 4096), (1000, 96), (37, 14336)])
+def test_both_index_paths(shape, dtype, hadamard, monkeypatch):
+    """Below 2^31 items the kernel splits an item index into (row, column) with a multiply-high by a
+    reciprocal the host computes; the kernel for larger tensors divides.  Both are forced here on row
+    lengths that are and are not powers of two, and must give the oracle's bytes."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(shape, generator=g).to(dtype)
+    for div64 in ("0", "1"):
+        monkeypatch.setenv("TB_QUANT_DIV64", div64)
+        _assert_same(x, hadamard)
+
+
+@pytest.mark.parametrize("hadamard", [False, True])
 def test_every_bf16_bit_pattern(hadamard):
     """All 65536 bf16 encodings (NaNs replaced by zero) under several block maxima."""
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)

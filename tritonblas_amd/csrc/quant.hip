@@ -13,6 +13,7 @@
 // This file is compiled with -ffp-contract=off: the rotation is fp32 adds/subs and one multiply.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include "quant.h"
 
 namespace tb {
@@ -150,7 +151,9 @@ static hipError_t launch_t(const QuantParams& p0, hipStream_t stream) {
   const int64_t items = p.m * nc;
   const int64_t per_block = 256 * UNROLL;
   const int64_t grid = (items + per_block - 1) / per_block;
-  if (items < (1ll << 31)) {
+  // testing hook: TB_QUANT_DIV64=1 takes the kernel for 2^31 items and more at any size
+  const char* env = getenv("TB_QUANT_DIV64");
+  if (items < (1ll << 31) && !(env && atoi(env))) {
     // floor(i / nc) for i < 2^31: with l = ceil(log2 nc) and magic = floor(2^(31+l) / nc) + 1 < 2^32,
     // (i * magic) >> (31 + l) is exact; the kernel takes the high product word and shifts by l - 1
     int l = 0;
