@@ -190,6 +190,13 @@ typedef struct tb_grouped_gemm_desc {
   const int32_t* group_offsets; /* device int32[num_groups+1], offsets[0]=0, offsets[g]=m_total     */
   int32_t block_m, block_n, block_k;
   int32_t group_m, num_xcds;
+  int32_t small_rows;         /* > 0: an expert's last, partial row block of at most this many rows is
+                                 left to a second launch with a short (32-row) tile instead of costing
+                                 a whole tall tile per column block.  0: library default — threshold 64,
+                                 and the kernels price both plans from the row counts on the device
+                                 (rounds of tall tiles against rounds of short ones) and split only
+                                 when that is cheaper; off when block_m is forced.  -1: one launch.
+                                 The split needs k % 256 == 0 and a tall (>= 128-row) tile.            */
 } tb_grouped_gemm_desc;
 
 int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* desc, void* stream);

@@ -109,6 +109,41 @@ def grouped_tile_lookup(tile_id, offsets, block_m, tiles_n):
     return None
 
 
+def grouped_two_launch_blocks(offsets, phase, big_m, small_rows, block_m):
+    """Row blocks (expert, first_row, end_row) of a grouped GEMM split over two launches: phase 1
+    tiles each expert's rows with big_m-row blocks but leaves a last partial block of at most
+    small_rows rows to phase 2, which tiles exactly those rows with block_m-row blocks.  Listed in the
+    table's order (experts ascending, blocks ascending).  New work, no reference counterpart."""
+    out = []
+    for e in range(len(offsets) - 1):
+        lo, hi = offsets[e], offsets[e + 1]
+        rows = max(hi - lo, 0)
+        full, rem = divmod(rows, big_m)
+        small = 0 < rem <= small_rows
+        if phase == 1:
+            mb = full + (1 if rem > 0 and not small else 0)
+            lim = lo + full * big_m if small else hi
+            out += [(e, lo + i * big_m, min(lo + (i + 1) * big_m, lim)) for i in range(mb)]
+        else:
+            base = lo + full * big_m
+            mb = cdiv(rem, block_m) if small else 0
+            out += [(e, base + i * block_m, min(base + (i + 1) * block_m, hi)) for i in range(mb)]
+    return out
+
+
+def grouped_split_pays(offsets, big_m, small_rows, small_m, tiles_n_big, tiles_n_small, grid_big, grid_small):
+    """The verdict both launches of a grouped GEMM reach on the device from the row counts: split when
+    2 * rounds(tall tiles of the split plan) + rounds(short tiles) < 2 * rounds(tall tiles of the
+    one-launch plan) and there is a short block at all (a round of short tiles streams half a tall
+    round's weight bytes and is priced at half its time).  New work, no reference counterpart."""
+    one = len(grouped_two_launch_blocks(offsets, 1, big_m, 0, big_m))
+    b1 = len(grouped_two_launch_blocks(offsets, 1, big_m, small_rows, big_m))
+    b2 = len(grouped_two_launch_blocks(offsets, 2, big_m, small_rows, small_m))
+    cost_one = 2 * cdiv(one * tiles_n_big, grid_big)
+    cost_two = 2 * cdiv(b1 * tiles_n_big, grid_big) + cdiv(b2 * tiles_n_small, grid_small)
+    return b2 > 0 and cost_two < cost_one
+
+
 def ws_global_atomic_tile(raw_idx, total_tiles, num_xcds):
     """Tile a work-stealing workgroup gets for counter value raw_idx in GLOBAL_ATOMIC mode
     (reference kernels/persistent_gemm_work_stealing.py:292-295, 321)."""

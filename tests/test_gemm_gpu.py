@@ -606,6 +606,28 @@ def test_fp4_fast_kernels_random_scales(tile, m, n, k):
 
 
 # ---- grouped MoE --------------------------------------------------------------------------------
+@pytest.mark.parametrize("small_rows", [-1, 32, 64, 100])
+@pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [0, 0, 5],
+                                    [256 + 33, 512 + 64, 65, 32, 768 + 100, 101]])
+def test_grouped_two_launches(counts, small_rows):
+    """Tall tiles forced, last partial row blocks of at most small_rows rows left to the second launch
+    with the 32-row tile: every row of C is written exactly once (C starts as NaN) with the oracle's
+    values, for thresholds on both sides of the remainders."""
+    import tritonblas_amd as tb
+    _say(f"grouped two launches counts={counts} small_rows={small_rows}")
+    E, n, k = len(counts), 384, 512
+    m = sum(counts)
+    offsets = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(14)).bfloat16()
+    w = torch.randn(E, n, k, generator=torch.Generator().manual_seed(10014)).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    wq, sw = OG.quantize_per_channel_fp8(w, axis=2)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda(), 256, 256, 128, small_rows=small_rows)
+    want = OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True)
+    _check(c.cpu(), want, torch.bfloat16, TOL_Q)
+
+
 @pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [0, 0, 5]])
 def test_grouped_a8w8(counts):
     import tritonblas_amd as tb

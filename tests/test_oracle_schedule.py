@@ -1,5 +1,6 @@
 """Brute-force checks of the integer schedule functions (CPU)."""
 import itertools
+import numpy as np
 
 import pytest
 
@@ -100,3 +101,39 @@ def test_grouped_tile_table():
            {(3, 0, nb) for nb in range(tn)}
     assert seen == want and t == len(want)
     assert t <= (S.cdiv(1024, bm) + 4) * tn   # the launch grid bound
+
+
+@pytest.mark.parametrize("small_rows", [1, 32, 64, 100, 255])
+def test_grouped_two_launches_cover_every_row_once(small_rows):
+    """Whatever the threshold, the two launches' row blocks partition every expert's rows, phase 2
+    only ever holds blocks of at most small_rows rows in total per expert, and both tables stay
+    inside the bounds the host sizes its grids with."""
+    rng = np.random.default_rng(small_rows)
+    for _ in range(50):
+        counts = [int(c) for c in rng.choice([0, 1, 5, 31, 32, 33, 64, 65, 100, 255, 256, 257, 300, 511, 512, 1030], size=rng.integers(1, 9))]
+        offsets = [0] + list(np.cumsum(counts))
+        big, bm2 = 256, 32
+        b1 = S.grouped_two_launch_blocks(offsets, 1, big, small_rows, big)
+        b2 = S.grouped_two_launch_blocks(offsets, 2, big, small_rows, bm2)
+        for e, c in enumerate(counts):
+            rows = sorted(r for (ee, a, b) in b1 + b2 if ee == e for r in range(a, b))
+            assert rows == list(range(offsets[e], offsets[e + 1]))
+            left = sum(b - a for (ee, a, b) in b2 if ee == e)
+            assert left == (c % big if 0 < c % big <= small_rows else 0)
+        assert all(0 < b - a <= big for _, a, b in b1) and all(0 < b - a <= bm2 for _, a, b in b2)
+        assert len(b1) <= S.cdiv(offsets[-1], big) + len(counts)
+        assert len(b2) <= len(counts) * S.cdiv(small_rows, bm2)
+
+
+def test_grouped_split_verdicts():
+    """Hand-priced cases on 256 compute units, 8 experts of (14336, 4096) weights: 56 column tiles of
+    256, 112 of 128.  Routed counts with five remainders of at most 27 rows: 37 blocks = 9 rounds
+    against 32 blocks = 7 rounds + 560 short tiles = 3 rounds (17 < 18: split).  Remainders of 60
+    rows on four experts: 36 blocks = 8 rounds (16) against 7 rounds + 896 short tiles = 4 rounds (18):
+    one launch.  Equal counts: nothing short, one launch."""
+    def verdict(counts):
+        return S.grouped_split_pays([0] + list(np.cumsum(counts)), 256, 64, 32, 56, 112, 256, 256)
+    assert verdict([1051, 1035, 1034, 1029, 997, 1019, 991, 1036]) is True
+    assert verdict([1084, 964] * 4) is False
+    assert verdict([1024] * 8) is False
+    assert verdict([8190, 1, 1, 0, 0, 0, 0, 0]) is True      # 34 blocks = 8 rounds (16) against 7 rounds + 1 (15)

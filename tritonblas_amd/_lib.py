@@ -78,7 +78,8 @@ class tb_grouped_gemm_desc(C.Structure):
                 ("a_stride_m", C.c_int64), ("w_stride_g", C.c_int64), ("w_stride_n", C.c_int64),
                 ("c_stride_m", C.c_int64), ("c_stride_n", C.c_int64), ("a_scale", C.c_void_p),
                 ("w_scale", C.c_void_p), ("group_offsets", C.c_void_p), ("block_m", C.c_int32),
-                ("block_n", C.c_int32), ("block_k", C.c_int32), ("group_m", C.c_int32), ("num_xcds", C.c_int32)]
+                ("block_n", C.c_int32), ("block_k", C.c_int32), ("group_m", C.c_int32), ("num_xcds", C.c_int32),
+                ("small_rows", C.c_int32)]
 
 
 class tb_quant_desc(C.Structure):

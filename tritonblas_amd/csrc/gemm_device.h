@@ -72,6 +72,15 @@ struct GemmParams {
   int32_t num_groups;
   int64_t b_group_stride;   // storage units between consecutive experts' weights
   int64_t sb_group_stride;  // floats
+  // grouped, two launches: phase 1 tiles every expert's rows with grp_big-row blocks but leaves a last
+  // partial block of at most grp_thr rows to phase 2, which tiles just those rows with a short tile
+  // (a handful of rows would otherwise cost a whole tall tile per column block).  Phase 0: one launch.
+  // With grp_auto every workgroup of both launches first prices the two plans from the row counts
+  // (rounds of tall tiles cost 2, rounds of short tiles 1) and both launches act on the same verdict:
+  // either the first runs the one-launch table and the second does nothing, or they split the rows.
+  int32_t grp_phase, grp_big, grp_thr;
+  int32_t grp_auto, grp_small_bm;
+  int32_t grp_other_tn, grp_other_grid;   // column tiles and grid of the other launch
 };
 
 struct TileCtx {
@@ -1083,18 +1092,46 @@ __device__ __forceinline__ void plain_tile(const GemmParams& p, int tile, int BM
   tc.B = p.B; tc.sb = p.sb;
 }
 
-// Grouped table: experts in order, expert e owns cdiv(rows_e, BM) * tiles_n tiles, m-block fastest.
-__device__ __forceinline__ bool grouped_tile(const GemmParams& p, int tile, int BM, int BN, int USZ, TileCtx& tc) {
+// Grouped table: experts in order, expert e owns (its row blocks in this phase) * tiles_n tiles, m-block fastest.
+// The phase this launch runs: 0 one-launch table, 1 / 2 the split tables, -1 nothing.
+__device__ __forceinline__ int grouped_phase(const GemmParams& p, int grid) {
+  if (p.grp_phase == 0 || !p.grp_auto) return p.grp_phase;
+  int b0 = 0, b1 = 0, b2 = 0;
+  for (int e = 0; e < p.num_groups; ++e) {
+    const int rows = max(p.group_offsets[e + 1] - p.group_offsets[e], 0);
+    const int full = rows / p.grp_big, rem = rows - full * p.grp_big;
+    const bool small = rem > 0 && rem <= p.grp_thr;
+    b0 += full + (rem > 0 ? 1 : 0);
+    b1 += full + ((rem > 0 && !small) ? 1 : 0);
+    b2 += small ? (rem + p.grp_small_bm - 1) / p.grp_small_bm : 0;
+  }
+  const int tn_big = p.grp_phase == 1 ? p.tiles_n : p.grp_other_tn, tn_small = p.grp_phase == 1 ? p.grp_other_tn : p.tiles_n;
+  const int g_big = p.grp_phase == 1 ? grid : p.grp_other_grid, g_small = p.grp_phase == 1 ? p.grp_other_grid : grid;
+  const int64_t one = 2 * (((int64_t)b0 * tn_big + g_big - 1) / g_big);
+  const int64_t two = 2 * (((int64_t)b1 * tn_big + g_big - 1) / g_big) + ((int64_t)b2 * tn_small + g_small - 1) / g_small;
+  const bool split = b2 > 0 && two < one;
+  if (p.grp_phase == 1) return split ? 1 : 0;
+  return split ? 2 : -1;
+}
+
+__device__ __forceinline__ bool grouped_tile(const GemmParams& p, int phase, int tile, int BM, int BN, int USZ, TileCtx& tc) {
   int acc = 0;
   for (int e = 0; e < p.num_groups; ++e) {
-    int lo = p.group_offsets[e], hi = p.group_offsets[e + 1];
-    int mb = (hi - lo + BM - 1) / BM;
-    int cnt = mb * p.tiles_n;
+    const int lo = p.group_offsets[e], hi = p.group_offsets[e + 1];
+    const int rows = max(hi - lo, 0);
+    int mb = (rows + BM - 1) / BM, base = lo, lim = hi;
+    if (phase != 0) {
+      const int full = rows / p.grp_big, rem = rows - full * p.grp_big;
+      const bool small = rem > 0 && rem <= p.grp_thr;
+      if (phase == 1) { mb = full + ((rem > 0 && !small) ? 1 : 0); if (small) lim = lo + full * p.grp_big; }
+      else { mb = small ? (rem + BM - 1) / BM : 0; base = lo + full * p.grp_big; }
+    }
+    const int cnt = mb * p.tiles_n;
     if (tile < acc + cnt) {
-      int local = tile - acc;
-      tc.m0 = lo + (local % mb) * BM;
+      const int local = tile - acc;
+      tc.m0 = base + (local % mb) * BM;
       tc.n0 = (local / mb) * BN;
-      tc.m_lim = hi; tc.n_lim = p.N;
+      tc.m_lim = lim; tc.n_lim = p.N;
       tc.B = p.B + (int64_t)e * p.b_group_stride * USZ;
       tc.sb = p.sb ? p.sb + (int64_t)e * p.sb_group_stride : nullptr;
       return true;
@@ -1111,9 +1148,11 @@ struct Sched {
   int step;               // work stealing: queue visit index
   int64_t start, last, q, rem;  // Stream-K iteration range of this workgroup
   int dp_tiles;
+  int gphase;             // grouped: which tile table this launch runs
 
   __device__ __forceinline__ void init(const GemmParams& p) {
     G = gridDim.x;
+    gphase = p.mode == MODE_GROUPED ? grouped_phase(p, G) : 0;
     pid = blockIdx.x;
     if (p.mode != MODE_WS && p.num_xcds > 1) pid = chiplet_transform_chunked(pid, G, p.num_xcds, p.chunk);
     next_tile = pid;
@@ -1140,8 +1179,8 @@ struct Sched {
     if (p.mode == MODE_GROUPED) {
       // the grid loops over the tile table; the first id past the table's end finishes the workgroup
       // (the host only knows an upper bound of the table's length)
-      if (next_tile >= p.total_tiles) return false;
-      bool ok = grouped_tile(p, next_tile, T::BM, T::BN, T::USZ, w.tc);
+      if (gphase < 0 || next_tile >= p.total_tiles) return false;
+      bool ok = grouped_tile(p, gphase, next_tile, T::BM, T::BN, T::USZ, w.tc);
       next_tile = ok ? next_tile + G : p.total_tiles;
       return ok;
     }

@@ -152,6 +152,7 @@ struct Job {
   // grouped
   const int32_t* group_offsets = nullptr; int num_groups = 0;
   int64_t b_group_stride = 0, sb_group_stride = 0;
+  int grp_phase = 0, grp_big = 0, grp_thr = 0, grp_auto = 0;   // see GemmParams
 };
 
 struct Plan {
@@ -307,7 +308,16 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     // the tile table has at most this many entries (every expert may end in a partial row block);
     // a resident grid loops over it
     p.mode = MODE_GROUPED;
-    const int64_t bound = ((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n;
+    p.grp_phase = j.grp_phase; p.grp_big = j.grp_big; p.grp_thr = j.grp_thr; p.grp_auto = j.grp_auto;
+    if (p.grp_phase == 1) {
+      // only a tall fast tile leaves its short last blocks to a second launch
+      if (v->fast && v->bm >= 128 && j.grp_thr > 0 && j.grp_thr < v->bm) p.grp_big = v->bm;
+      else p.grp_phase = 0;
+    }
+    if (p.grp_phase == 2 && (p.grp_big <= 0 || p.grp_thr <= 0)) return TB_ERR_BAD_ARGUMENT;
+    const int64_t bound = p.grp_phase == 2
+        ? (int64_t)j.num_groups * ((j.grp_thr + v->bm - 1) / v->bm) * p.tiles_n
+        : ((j.M + v->bm - 1) / v->bm + j.num_groups) * p.tiles_n;
     if (bound > INT32_MAX) return TB_ERR_BAD_SHAPE;
     p.total_tiles = (int32_t)bound;
     grid = (int)std::min<int64_t>(bound, resident);
@@ -376,6 +386,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   return TB_OK;
 }
 
+int run_plan(const Job& j, Plan& plan, hipStream_t stream);
+
 int launch(const Job& j, hipStream_t stream) {
   tb_hw hw;
   int st = current_hw(&hw);
@@ -383,6 +395,10 @@ int launch(const Job& j, hipStream_t stream) {
   Plan plan;
   st = make_plan(j, hw, true, &plan);
   if (st != TB_OK) return st;
+  return run_plan(j, plan, stream);
+}
+
+int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
   GemmParams& p = plan.p;
   if (plan.skinny) {
     if (launch_skinny(p, j.dt, stream) != hipSuccess) { (void)hipGetLastError(); return TB_ERR_LAUNCH; }
@@ -556,6 +572,9 @@ int tb_gemm_fp4(const tb_gemm_fp4_desc* d, void* stream) {
   return launch(j, (hipStream_t)stream);
 }
 
+// the short FP8 tile the second launch of a grouped GEMM runs
+constexpr int kGroupedSmallBM = 32, kGroupedSmallBN = 128, kGroupedSmallBK = 256;
+
 int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_grouped_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
@@ -573,7 +592,33 @@ int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
   j.group_offsets = d->group_offsets; j.num_groups = d->num_groups;
   j.b_group_stride = d->w_stride_g; j.sb_group_stride = d->n;
   if ((d->w_stride_g * 1) % 16) return TB_ERR_BAD_LAYOUT;
-  return launch(j, (hipStream_t)stream);
+  // Two launches unless switched off or a tile is forced: tall tiles for whole row blocks and long
+  // remainders, then a short streaming tile for the experts whose last block holds few rows (the row
+  // counts live on the device, so both tile tables are evaluated there; an empty second table costs
+  // one empty launch).
+  if (d->small_rows < -1) return TB_ERR_BAD_ARGUMENT;
+  const int thr = d->small_rows > 0 ? d->small_rows : 64;
+  const bool two = d->small_rows > 0 || (d->small_rows == 0 && d->block_m == 0);
+  if (!two || d->k % kGroupedSmallBK) return launch(j, (hipStream_t)stream);
+  j.grp_phase = 1; j.grp_thr = thr; j.grp_auto = d->small_rows == 0;
+  tb_hw hw;
+  int st = current_hw(&hw);
+  if (st != TB_OK) return st;
+  Plan first, second;
+  st = make_plan(j, hw, true, &first);
+  if (st != TB_OK) return st;
+  if (first.p.grp_phase != 1) return run_plan(j, first, (hipStream_t)stream);
+  Job j2 = j;
+  j2.bm = kGroupedSmallBM; j2.bn = kGroupedSmallBN; j2.bk = kGroupedSmallBK;
+  j2.grp_phase = 2; j2.grp_big = first.p.grp_big;
+  st = make_plan(j2, hw, true, &second);
+  if (st != TB_OK) return st;
+  first.p.grp_small_bm = second.p.grp_small_bm = second.v->bm;
+  first.p.grp_other_tn = second.p.tiles_n; first.p.grp_other_grid = second.grid;
+  second.p.grp_other_tn = first.p.tiles_n; second.p.grp_other_grid = first.grid;
+  st = run_plan(j, first, (hipStream_t)stream);
+  if (st != TB_OK) return st;
+  return run_plan(j2, second, (hipStream_t)stream);
 }
 
 int tb_hadamard_mxfp4_quant(const tb_quant_desc* d, void* stream) {

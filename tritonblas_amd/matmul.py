@@ -360,10 +360,12 @@ def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = 
 
 
 def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int = None, block_n: int = None,
-                        block_k: int = None):
+                        block_k: int = None, small_rows: int = 0):
     """Grouped (MoE) FP8 GEMM: rows ``group_offsets[e]:group_offsets[e+1]`` of ``a`` (M, K) meet expert
     weight ``w[e]`` (N, K); ``c[rows] = cast((a[rows] @ w[e].T) * a_scale[rows, None] * w_scale[e][None, :])``.
-    ``group_offsets`` is an int32 device tensor of E+1 ascending row offsets.  One launch, no host sync."""
+    ``group_offsets`` is an int32 device tensor of E+1 ascending row offsets.  No host sync: the row counts
+    are only read on the device.  An expert's last partial row block of at most ``small_rows`` rows goes to a
+    second launch with a 32-row tile (0: the library's default of 64 rows, off when a tile is forced; -1: off)."""
     M, K = a.shape
     E, N, K2 = w.shape
     assert K == K2 and c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
@@ -386,6 +388,7 @@ def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int =
     d.group_offsets = _ptr(group_offsets)
     if block_m is not None:
         d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
+    d.small_rows = small_rows
     with _on_device(dev):
         _lib.check(_lib.load().tb_grouped_gemm_fp8(d, _lib.stream_handle(dev)), "tb_grouped_gemm_fp8")
     return c
