@@ -8,12 +8,14 @@ Follows the reference's Triton quantiser bit by bit
 rotation has no counterpart in the reference; it is defined here by a pinned
 butterfly order and checked against the Sylvester matrix.
 
-Spec decisions for inputs the reference leaves to GPU behaviour (documented,
-not pinned by any reference fixture):
+Decisions for inputs whose treatment the reference's source leaves to the platform:
   * scale byte = (e + 127) mod 256, so an all-zero block stores byte 0;
   * shifts by >= 32 in the sub-normal mantissa path give 0;
   * log2/exp2 of powers of two are exact integer exponent arithmetic;
   * NaN inputs are unspecified.
+The first three agree with what the reference kernel itself produces under Triton's CPU interpreter
+(tests/golden/mxfp4_quant_vectors.npz holds such blocks, fp32 denormals and infinities included);
+what a GPU build of the reference does there is not pinned by anything in the reference tree.
 """
 import numpy as np
 

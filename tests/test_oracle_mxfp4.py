@@ -137,3 +137,28 @@ def test_rotated_gemm_preserved():
     a = rng.standard_normal((4, 64)).astype(np.float32)
     b = rng.standard_normal((5, 64)).astype(np.float32)
     assert np.allclose(mxfp4.hadamard32(a) @ mxfp4.hadamard32(b).T, a @ b.T, atol=1e-4)
+
+
+def _reference_vectors():
+    """tests/golden/mxfp4_quant_vectors.npz: outputs of the reference's own kernel
+    (include/tritonblas/utils.py:646-789), run under Triton's CPU interpreter by
+    tests/golden/make_mxfp4_quant_vectors.py."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mxfp4_quant_vectors.npz"))
+    x32 = d["x_f32_bits"].view(np.float32)
+    xbf = (d["x_bf16_bits"].astype(np.uint32) << 16).view(np.float32)
+    return {"f32": (x32, d["codes_f32"], d["scales_f32"]), "bf16": (xbf, d["codes_bf16"], d["scales_bf16"])}
+
+
+@pytest.mark.parametrize("name", ["f32", "bf16"])
+def test_oracle_equals_reference_kernel_output(name):
+    """Every code byte and scale byte of the reference kernel's output, including the cases its source
+    leaves to the platform: scale bytes of negative exponents, all-zero blocks (byte 0), denormal block
+    maxima, shift counts of 32 and more, infinities."""
+    x, codes, scales = _reference_vectors()[name]
+    got_c, got_s = mxfp4.mxfp4_quant(x)
+    assert np.array_equal(got_s, scales)
+    assert np.array_equal(got_c, codes)
+    # the set is not trivial: many scale bytes on both sides of the bias, zero blocks, every code
+    assert len(np.unique(scales)) > 60 and scales.min() == 0 and scales.max() > 250
+    assert set(np.unique(mxfp4.unpack_codes(codes))) == set(range(16))

@@ -54,6 +54,22 @@ def test_both_index_paths(shape, dtype, hadamard, monkeypatch):
         _assert_same(x, hadamard)
 
 
+@pytest.mark.parametrize("name", ["f32", "bf16"])
+def test_reference_kernel_vectors(name):
+    """The HIP quantiser against the committed outputs of the reference's own kernel
+    (tests/golden/mxfp4_quant_vectors.npz, written by tests/golden/make_mxfp4_quant_vectors.py from
+    include/tritonblas/utils.py:646-789 under Triton's CPU interpreter): bit for bit."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mxfp4_quant_vectors.npz"))
+    if name == "f32":
+        x = torch.from_numpy(d["x_f32_bits"].view(np.float32).copy())
+    else:
+        x = torch.from_numpy(d["x_bf16_bits"].view(np.int16).copy()).view(torch.bfloat16)
+    got_c, got_s = _run(x, False)
+    assert np.array_equal(got_s, d[f"scales_{name}"]), f"{(got_s != d[f'scales_{name}']).sum()} scale bytes differ"
+    assert np.array_equal(got_c, d[f"codes_{name}"]), f"{(got_c != d[f'codes_{name}']).sum()} code bytes differ"
+
+
 @pytest.mark.parametrize("hadamard", [False, True])
 def test_every_bf16_bit_pattern(hadamard):
     """All 65536 bf16 encodings (NaNs replaced by zero) under several block maxima."""
