@@ -135,8 +135,10 @@ def _grouped_cases(n, seed):
     for i in range(n):
         experts = rng.randint(1, 9)
         counts = [rng.choice([0, 1, rng.randint(1, 70), rng.randint(100, 600), 256, 257]) for _ in range(experts)]
-        out.append(dict(idx=i, counts=counts, n=rng.choice([64, 200, 384, 1000]), k=rng.choice([128, 512, 1152]),
-                        seed=rng.randint(0, 1 << 30)))
+        # plan: the library's own (0: one or two launches, priced on the device), one launch (-1), or the
+        # tall tile forced and last row blocks of at most that many rows left to the second launch
+        out.append(dict(idx=i, counts=counts, n=rng.choice([64, 200, 384, 1000]), k=rng.choice([128, 512, 1152, 1024]),
+                        seed=rng.randint(0, 1 << 30), small_rows=rng.choice([0, 0, -1, 16, 32, 64, 100, 200])))
     return out
 
 
@@ -158,7 +160,8 @@ def test_random_grouped_case(case):
     aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
     wq, sw = OG.quantize_per_channel_fp8(w, axis=2)
     c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-    tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda())
+    tile = (256, 256, 128) if case["small_rows"] > 0 else (None, None, None)
+    tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda(), *tile, small_rows=case["small_rows"])
     want = OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True)
     got = c.cpu()
     assert torch.isfinite(got.float()).all()
