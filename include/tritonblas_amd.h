@@ -145,6 +145,12 @@ typedef struct tb_gemm_desc {
   int32_t ws_local_tiles_per_xcd, ws_global_tiles;  /* TB_WS_HIERARCHICAL: both 0 = split by the
                                  reference's rule (tb_hierarchical_split) for the tile the launch
                                  runs; otherwise num_xcds * local + global must equal its tile count */
+  int32_t column_split;       /* persistent schedule, tiles that do not fill a whole number of rounds of
+                                 the resident grid: 0 = the library may run the columns that fill whole
+                                 rounds with the given tile and the remaining columns as a second launch
+                                 with the tile its model picks for them (when the model expects at least
+                                 3 % from it; disjoint column ranges of C, same stream); -1 = one launch.
+                                 No counterpart in the reference.                                       */
 } tb_gemm_desc;
 
 /* C = cast((A @ B) * a_scale[:,None] * b_scale[None,:] + bias[None,:]), fp32 accumulate.

@@ -605,6 +605,49 @@ def test_fp4_fast_kernels_random_scales(tile, m, n, k):
     _check(c.cpu(), OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True), torch.float32, 1e-5)
 
 
+# ---- column split of a partial last round -----------------------------------------------------------
+@pytest.mark.parametrize("kind", ["fp8", "bf16", "bias"])
+@pytest.mark.parametrize("shape", [(2048, 28672, 512), (1536, 14336 + 40, 256), (1100, 20000, 384)])
+def test_column_split(kind, shape, monkeypatch):
+    """More tiles than the resident grid holds and a partial last round: the library may run the columns
+    that fill whole rounds with the selected tile and the rest as a second launch with another tile.
+    Forced here; every element of C must equal the one-launch result bit for bit (each output element
+    sums its K range in the same order whatever tile it sits in), and a strip across the seam is
+    checked against the oracle."""
+    import tritonblas_amd as tb
+    m, n, k = shape
+    _say(f"column split {kind} {m}x{n}x{k}")
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(n, k, generator=g).bfloat16()
+    bias = torch.randn(n, generator=g).bfloat16() if kind == "bias" else None
+    outs = {}
+    for name, env in (("one", {"TB_NO_COLUMN_SPLIT": "1", "TB_FORCE_COLUMN_SPLIT": "0"}), ("split", {"TB_NO_COLUMN_SPLIT": "0", "TB_FORCE_COLUMN_SPLIT": "1"})):
+        for key, val in env.items():
+            monkeypatch.setenv(key, val)
+        c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        # the tall tile named outright, so that the tile count (and with it the seam) is known
+        import types
+        sel = types.SimpleNamespace(block_m=256, block_n=256, block_k=128 if kind == "fp8" else 64, group_m=min(8, -(-m // 256)),
+                                    num_sms=8, COUNTERS_PER_XCD=1, streamk=False, sk_grid=0, _total_cus=None, waves_per_eu=1)
+        if kind == "fp8":
+            aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+            wq, sw = OG.quantize_per_channel_fp8(w, axis=1)
+            tb.matmul_a8w8_lt(aq.cuda(), wq.cuda().T, sa.cuda(), sw.cuda(), c, sel, None)
+        else:
+            from tritonblas_amd.matmul import persistent_matmul_lt
+            persistent_matmul_lt(a.cuda(), w.cuda().T, c, sel, None, bias=None if bias is None else bias.cuda())
+        outs[name] = c.cpu()
+    assert torch.isfinite(outs["split"].float()).all()
+    assert torch.equal(outs["one"], outs["split"])
+    cols = slice(n // 2, n)     # the seam lies in the right half (whole rounds come first)
+    if kind == "fp8":
+        want = OG.ref_gemm(aq, wq.T[:, cols], torch.float32, a_scale=sa, b_scale=sw[cols])
+    else:
+        want = OG.ref_gemm(a, w.T[:, cols], torch.float32, bias=None if bias is None else bias[cols])
+    _check(outs["split"][:, cols], want, torch.bfloat16, TOL_Q if kind == "fp8" else TOL_16)
+
+
 # ---- grouped MoE --------------------------------------------------------------------------------
 @pytest.mark.parametrize("small_rows", [-1, 32, 64, 100])
 @pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [0, 0, 5],

@@ -58,7 +58,7 @@ class tb_gemm_desc(C.Structure):
                 ("counters_per_xcd", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
                 ("epoch", C.c_uint32), ("spin_limit", C.c_uint32), ("cu_mask", C.c_void_p),
                 ("cu_mask_len", C.c_int32), ("ws_mode", C.c_int32), ("ws_local_tiles_per_xcd", C.c_int32),
-                ("ws_global_tiles", C.c_int32)]
+                ("ws_global_tiles", C.c_int32), ("column_split", C.c_int32)]
 
 
 class tb_gemm_fp4_desc(C.Structure):

@@ -153,6 +153,7 @@ struct Job {
   const int32_t* group_offsets = nullptr; int num_groups = 0;
   int64_t b_group_stride = 0, sb_group_stride = 0;
   int grp_phase = 0, grp_big = 0, grp_thr = 0, grp_auto = 0;   // see GemmParams
+  int column_split = 0;
 };
 
 struct Plan {
@@ -418,6 +419,60 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
   return TB_OK;
 }
 
+// Persistent schedule with a partial last round: a resident grid of G workgroups needs ceil(tiles / G)
+// rounds however few tiles the last one holds.  When the model expects it to pay, the columns that fill
+// whole rounds run with the planned tile and the remaining columns as a problem of their own, with the
+// tile the model picks for them (usually a smaller one that spreads over all CUs).  Both launches write
+// disjoint column ranges of C on the same stream.
+int launch_columns(const Job& j, hipStream_t stream) {
+  const char* off = getenv("TB_NO_COLUMN_SPLIT");
+  if (j.schedule != TB_SCHED_PERSISTENT || j.column_split != 0 || j.grid > 0 || j.num_groups > 0 || (off && atoi(off)))
+    return launch(j, stream);
+  tb_hw hw;
+  int st = current_hw(&hw);
+  if (st != TB_OK) return st;
+  Plan whole;
+  st = make_plan(j, hw, true, &whole);
+  if (st != TB_OK) return st;
+  const Variant* v = whole.v;
+  const int64_t total = whole.p.total_tiles, G = whole.grid, tiles_m = whole.p.tiles_m, tiles_n = whole.p.tiles_n;
+  if (whole.skinny || whole.p.mode != MODE_STATIC || !v->fast || total <= G || total % G == 0) return run_plan(j, whole, stream);
+  const int64_t tn1 = (total / G) * G / tiles_m;
+  if (tn1 <= 0 || tn1 >= tiles_n) return run_plan(j, whole, stream);
+  const int64_t n1 = tn1 * v->bn, n2 = j.N - n1;
+  tb_problem pr;
+  std::memset(&pr, 0, sizeof(pr));
+  pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+  pr.a_k_contiguous = pr.b_k_contiguous = 1;
+  const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, v->minb, v->fast, v->stages};
+  const double t_whole = estimate_tile_us(pr, hw, ti, false);
+  pr.n = n1;
+  const double t_first = estimate_tile_us(pr, hw, ti, false);
+  pr.n = n2;
+  tb_selection rest;
+  auto infos = tile_infos(j.dt);
+  if (select_tile(pr, hw, infos.data(), (int)infos.size(), &rest) != TB_OK) return run_plan(j, whole, stream);
+  // (testing hook: TB_FORCE_COLUMN_SPLIT=1 splits whatever the model says)
+  const char* force = getenv("TB_FORCE_COLUMN_SPLIT");
+  if (!(force && atoi(force)) && t_first + rest.est_total_us > 0.97 * t_whole) return run_plan(j, whole, stream);
+  const int usz = unit_bytes(j.dt);
+  Job a = j, b = j;
+  a.N = n1; a.bm = v->bm; a.bn = v->bn; a.bk = v->bk;
+  b.N = n2; b.bm = b.bn = b.bk = 0; b.group_m = 0;
+  b.B = (const uint8_t*)j.B + n1 * j.b_sr * usz;
+  b.C = (uint8_t*)j.C + n1 * j.c_sn * c_bytes(j.c_type);
+  if (j.sb) b.sb = j.sb + n1;
+  if (j.bias) b.bias = (const uint8_t*)j.bias + n1 * j.bias_stride * (j.bias_type == TB_F32 ? 4 : 2);
+  if (j.mxb) b.mxb = (const uint8_t*)j.mxb + n1 * j.mxb_sr;
+  Plan pa, pb;
+  st = make_plan(a, hw, true, &pa);
+  if (st == TB_OK) st = make_plan(b, hw, true, &pb);
+  if (st != TB_OK || pa.v != v) return run_plan(j, whole, stream);   // (the split must not change what the main part runs)
+  st = run_plan(a, pa, stream);
+  if (st != TB_OK) return st;
+  return run_plan(b, pb, stream);
+}
+
 int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
@@ -436,6 +491,7 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   j->workspace = d->workspace; j->workspace_bytes = d->workspace_bytes; j->epoch = d->epoch; j->spin_limit = d->spin_limit;
   j->cu_mask = d->cu_mask; j->cu_mask_len = d->cu_mask_len; j->ws_mode = d->ws_mode;
   j->ws_local = d->ws_local_tiles_per_xcd; j->ws_global = d->ws_global_tiles;
+  j->column_split = d->column_split;
   return TB_OK;
 }
 
@@ -539,7 +595,8 @@ int tb_gemm(const tb_gemm_desc* desc, void* stream) {
   int st = job_from_gemm(desc, &j);
   if (st != TB_OK) return st;
   if (!j.A || !j.B || !j.C) return TB_ERR_NULL_POINTER;
-  return launch(j, (hipStream_t)stream);
+  if (desc->column_split < -1 || desc->column_split > 0) return TB_ERR_BAD_ARGUMENT;
+  return launch_columns(j, (hipStream_t)stream);
 }
 
 size_t tb_workspace_bytes(const tb_gemm_desc* desc) {
