@@ -116,6 +116,30 @@ def test_selector_properties_and_lds_fit():
             assert s.COUNTERS_PER_XCD == O.ws_counters_per_xcd(total)
 
 
+def test_streamk_whole_tiles_answer_survives_the_resident_clamp():
+    """FP8 2048x14336x4096 with 256x256 tiles: 448 tiles on 256 resident workgroups, and the model says
+    that a second round of whole tiles beats a shared tail (its answer is the tile count, 448).  A
+    launch that asks for that grid, or for none, must then run whole tiles only -- which shows as a
+    Stream-K descriptor that needs no workspace -- and not a 256-workgroup grid with 192 shared tiles."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    m, n, k = 2048, 14336, 4096
+    s = tb.OrigamiMatmulSelector(m, n, k, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.bfloat16, torch.device("cuda"), streamk=True)
+    assert (s.block_m, s.block_n) == (256, 256) and s.sk_grid == 448
+    for grid in (0, 448):
+        d = _lib.tb_gemm_desc()
+        d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+        d.a_type = d.b_type = _lib.tb_dtype(torch.float8_e4m3fn)
+        d.c_type = _lib.tb_dtype(torch.bfloat16)
+        d.m, d.n, d.k = m, n, k
+        d.a_stride_m, d.a_stride_k, d.b_stride_n, d.b_stride_k, d.c_stride_m, d.c_stride_n = k, 1, k, 1, n, 1
+        d.block_m, d.block_n, d.block_k = 256, 256, 128
+        d.schedule, d.grid = _lib.TB_SCHED_STREAMK, grid
+        assert _lib.load().tb_workspace_bytes(d) == 0
+    d.grid = 256      # an explicit resident grid still shares the 192-tile tail
+    assert _lib.load().tb_workspace_bytes(d) > 256 * 256 * 256 * 4
+
+
 def test_argument_validation_without_a_gpu():
     from tritonblas_amd import _lib
     lib = _lib.load()

@@ -102,12 +102,16 @@ static double family_efficiency(int dt, const TileInfo& v) {
 //     unless another round of whole tiles is expected to be as fast (large tiles have expensive partial
 //     tiles: 2048x14336x4096 bf16, 448 tiles of 256x256 on 256 slots: 209 us in two rounds, 253 us with a
 //     shared tail); the return value `total` means "whole tiles only".
+static const double kSharedTailFactor = 4.0;
 int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us) {
   if (total <= 0 || slots <= 0) return 1;
   if (total >= slots) {
     const int64_t tail = total % slots;
     if (tail == 0) return slots;
-    const double shared = std::ceil((double)tail * k_iters / slots) * step_us + (std::ceil((double)slots / tail) - 1.0) * fix_us;
+    // (a tail shared by the whole grid costs about four times the per-segment figure that the split of
+    // a few tiles shows: 2048x28672x8192 FP8, 128 tiles of 256x256 shared by 256 workgroups, ~100 us on
+    // top of their K steps; 1024x28672x8192, 192 shared tiles, the same)
+    const double shared = std::ceil((double)tail * k_iters / slots) * step_us + (std::ceil((double)slots / tail) - 1.0) * fix_us * kSharedTailFactor;
     const double whole = (double)k_iters * step_us;
     return shared < whole ? slots : (int)std::min<int64_t>(total, INT32_MAX);
   }
@@ -168,7 +172,8 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
       if (tail > 0) {
         const double iters = std::ceil((double)tail * k_iters / grid);
         const double segments = std::ceil((double)grid / tail);
-        us += iters * t_step + (segments - 1.0) * fix_us + t_tile;
+        // (tiles < grid: every tile is cut into `segments` pieces; otherwise a tail shared by the whole grid)
+        us += iters * t_step + (segments - 1.0) * fix_us * (dp_rounds > 0 ? kSharedTailFactor : 1.0) + t_tile;
       }
     }
   } else {

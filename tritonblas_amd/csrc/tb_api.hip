@@ -360,7 +360,9 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       tb_hw hw_res = hw;   // (what the model may fill: the kernel's real occupancy)
       const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, occ, v->fast, v->stages};
       g = streamk_grid_for(pr, hw_res, ti);
-      if (g > resident) g = resident;
+      // (the model's "whole tiles only" answer is the tile count itself and must survive the clamp)
+      if (g >= total) g = total;
+      else if (g > resident) g = resident;
     }
     const bool whole_only = g == total;   // exactly one workgroup per tile (however many fit at once): nothing to share
     if (whole_only) g = std::min<int64_t>(total, resident);
