@@ -5,6 +5,8 @@
 namespace tb {
 
 const Variant g_variants_fp8[] = {
+    // hand-scheduled 4-wave kernel: taken when K is a multiple of two K steps and no Stream-K tail is asked for
+    make_variant_w4<W4Tile<DT_FP8>>(),
     make_variant<Tile<DT_FP8, 256, 256, 128, 2, 4, LAY_K, LAY_K, 1, true, 2>>(),
     make_variant<Tile<DT_FP8, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_FP8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),

@@ -2,6 +2,7 @@
 #pragma once
 #include <stdint.h>
 #include "gemm_device.h"
+#include "gemm_w4.h"
 
 namespace tb {
 
@@ -11,13 +12,21 @@ struct Variant {
   int wm, wn, threads, lds_bytes, minb;
   int fast, stages;       // fast: vector/LDS-direct loaders (alignment + K multiple required)
   const void* kernel;     // __global__ void (*)(const GemmParams), whole-tile schedules
-  const void* kernel_sk;  // same tile with the Stream-K tail
+  const void* kernel_sk;  // same tile with the Stream-K tail (null: this variant has none)
+  int k_step_pairs;       // 1: hand-scheduled 4-wave kernel -- K must be a multiple of two K steps
 };
 
 template <class T>
 constexpr Variant make_variant() {
   return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_ALLOC, T::MINB,
-                 T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>};
+                 T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>, 0};
+}
+
+// the hand-scheduled 4-wave kernel of gemm_w4.h for the same tile shape
+template <class T>
+constexpr Variant make_variant_w4() {
+  return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_ALLOC, 1,
+                 1, T::STAGES, (const void*)&gemm_kernel_w4<T>, nullptr, 1};
 }
 
 // defined one per translation unit

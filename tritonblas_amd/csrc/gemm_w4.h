@@ -1,0 +1,258 @@
+// 256x256 tile GEMM with four waves (one per SIMD), 128x128 wave tiles and a hand-scheduled K loop.
+//
+// The compiler-scheduled kernels of gemm_device.h run the 256x256 tile with eight waves (128x64 wave
+// tiles): with one wave per SIMD every LDS wait of compiler-ordered code stalls the only wave there is,
+// and 256 accumulator registers leave the allocator no room.  Here the K loop of one output tile is one
+// assembly statement (gen_w4.py writes it): the accumulators live in a[0:255], fragments and scales
+// in v[0:191], every MFMA, LDS read, LDS-direct copy and wait is placed by hand.  Everything around
+// it -- tile schedule, per-tile addresses, epilogue -- stays C++.  The wave tile is a quarter of the
+// 8-wave kernels' K-step LDS traffic less (128 KB instead of 196 KB of fragment reads per 64 KB copied).
+//
+// Differences from the 8-wave kernels that matter to callers: K must be a multiple of two K steps and
+// there is no Stream-K variant (whole tiles only: data-parallel, work-stealing and grouped schedules).
+// Sums are formed in the same order (same MFMA instruction, same K grouping, K steps in ascending
+// order), so results are bit-identical to the 8-wave kernels'.
+//
+// Output layout.  The B tile is the first MFMA operand, so a lane holds four consecutive output
+// columns of one row per MFMA tile.  The rows of the B tile are copied into LDS in a permuted order
+// (LDS row 16j + 4g + e of a wave's 128 holds column 32(j/2) + 8g + 4(j%2) + e), which makes the eight
+// values a lane holds for MFMA tiles 2q and 2q+1 eight consecutive columns: the epilogue stores them
+// as one 16-byte write per lane straight from registers (64 contiguous bytes per row and instruction),
+// with no LDS staging -- the LDS already belongs to the next tile's first K steps by then.
+#pragma once
+#include <utility>
+#include "gemm_device.h"
+
+namespace tb {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// accumulator register a[N] (written by the K loop statement; the compiler never allocates these)
+template <int N>
+__device__ __forceinline__ float acc_read() {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
+  return x;
+}
+
+template <int DT>
+using W4Tile = Tile<DT, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>;
+
+// what the K loop needs to know about one output tile
+struct W4TileArgs {
+  const uint8_t* A;      // first row of the tile, k = 0
+  const uint8_t* B;
+  const uint8_t* mxa;    // FP4: scale rows
+  const uint8_t* mxb;
+  v16i off;              // byte offsets of this lane's 8 + 8 copy chunks from (A, B) at a K step's origin
+  uint32_t sca, scb;     // FP4: byte offsets of this lane's scale rows from (mxa, mxb)
+};
+
+struct W4Lane {
+  int r, g, wm0, wn0;
+  uint32_t c16;          // swizzled chunk (byte offset) this lane copies in every row it copies
+  int pa, pb;            // tile row this lane copies with copy instruction 0 (instruction i: + 32 i)
+  int sra, srb;          // FP4: tile rows whose scales this lane copies
+};
+
+template <class T>
+__device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, W4TileArgs& t) {
+  const int rva = tc.m_lim - tc.m0, rvb = tc.n_lim - tc.n0;
+  const uint32_t sra = (uint32_t)p.a_sr, srb = (uint32_t)p.b_sr;   // bytes (one-byte storage units)
+  t.A = p.A + (int64_t)tc.m0 * p.a_sr;
+  t.B = tc.B + (int64_t)tc.n0 * p.b_sr;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    t.off[i] = (int)((uint32_t)min(i * 32 + ln.pa, rva - 1) * sra + ln.c16);
+    t.off[8 + i] = (int)((uint32_t)min(i * 32 + ln.pb, rvb - 1) * srb + ln.c16);
+  }
+  if constexpr (T::DT == DT_FP4) {
+    t.mxa = p.mxa + (int64_t)tc.m0 * p.mxa_sr;
+    t.mxb = p.mxb + (int64_t)tc.n0 * p.mxb_sr;
+    t.sca = (uint32_t)min(ln.sra, rva - 1) * (uint32_t)p.mxa_sr;
+    t.scb = (uint32_t)min(ln.srb, rvb - 1) * (uint32_t)p.mxb_sr;
+  } else {
+    t.mxa = t.mxb = nullptr;
+    t.sca = t.scb = 0;
+  }
+}
+
+// acc * (sa*sb) + bias -> cast -> store, straight from the accumulator registers.  Lane (g, r) of wave
+// (wm, wn) holds, for row block i and column group q, C[m0 + wm0 + 16i + r][n0 + wn0 + 32q + 8g + 0..7].
+template <class T, int CT>
+__device__ __forceinline__ void epilogue_w4(const GemmParams& p, const TileCtx& tc, const W4Lane& ln) {
+  float sav[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = tc.m0 + ln.wm0 + i * 16 + ln.r;
+    sav[i] = (p.sa && m < tc.m_lim) ? p.sa[m] : 1.f;
+  }
+  static_for<4>([&](auto Q) {
+    constexpr int q = decltype(Q)::value;
+    const int n = tc.n0 + ln.wn0 + 32 * q + 8 * ln.g;
+    const int nvalid = tc.n_lim - n;
+    float sbv[8], bv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sbv[e] = (tc.sb && e < nvalid) ? tc.sb[n + e] : 1.f;
+      bv[e] = (p.bias && e < nvalid)
+                  ? load_as_f32(p.bias + (int64_t)(n + e) * p.bias_stride * (p.bias_type == DT_F32 ? 4 : 2), p.bias_type)
+                  : 0.f;
+    }
+    static_for<8>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      float v[8];
+      static_for<8>([&](auto E) {
+        constexpr int e = decltype(E)::value;
+        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3))>();
+      });
+      const int m = tc.m0 + ln.wm0 + i * 16 + ln.r;
+      if (m >= tc.m_lim || nvalid <= 0) return;
+      if (p.sa) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * (sav[i] * sbv[e]);
+      }
+      if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] + bv[e];
+      }
+      if constexpr (CT == DT_F32) {
+        float* cp = (float*)p.C + ((int64_t)m * p.c_sm + (int64_t)n * p.c_sn);
+        if (p.c_line && nvalid >= 8) {
+          const v4f lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+          if (p.c_nt) { __builtin_nontemporal_store(lo, (v4f*)cp); __builtin_nontemporal_store(hi, (v4f*)cp + 1); }
+          else { *(v4f*)cp = lo; *((v4f*)cp + 1) = hi; }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (e < nvalid) cp[e * p.c_sn] = v[e];
+        }
+      } else {
+        uint32_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if constexpr (CT == DT_F16) h[e] = __builtin_bit_cast(uint16_t, (_Float16)v[e]);
+          else h[e] = __builtin_bit_cast(uint16_t, (__bf16)v[e]);
+        }
+        uint16_t* cp = (uint16_t*)p.C + ((int64_t)m * p.c_sm + (int64_t)n * p.c_sn);
+        if (p.c_line && nvalid >= 8) {
+          const v4i pk = {(int)(h[0] | (h[1] << 16)), (int)(h[2] | (h[3] << 16)), (int)(h[4] | (h[5] << 16)), (int)(h[6] | (h[7] << 16))};
+          if (p.c_nt) __builtin_nontemporal_store(pk, (v4i*)cp);
+          else *(v4i*)cp = pk;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (e < nvalid) cp[e * p.c_sn] = (uint16_t)h[e];
+        }
+      }
+    });
+  });
+}
+
+template <class T>
+__global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
+  static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
+  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4, "element types with a 128-byte K step per MFMA");
+  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_ALLOC];
+  int& s_bcast = *(int*)(lds + T::LDS_ALLOC - 16);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds);
+
+  W4Lane ln;
+  ln.r = lane & 15;
+  ln.g = lane >> 4;
+  ln.wm0 = (wave >> 1) * 128;
+  ln.wn0 = (wave & 1) * 128;
+  const int l8 = lane >> 3;
+  // copy instruction i of this wave fills LDS rows 32i + 8*wave + l8 (A rows, then B rows), chunk slot
+  // lane % 8; the row's swizzle mask is (row % 8) ^ ((row / 8) & 1) = l8 ^ (wave & 1)
+  ln.c16 = (uint32_t)(((lane & 7) ^ l8 ^ (wave & 1)) << 4);
+  ln.pa = wave * 8 + l8;
+  // B: LDS row rho = 16j + 4g' + e (within a wave's 128 rows) takes tile row 32(j/2) + 8g' + 4(j%2) + e
+  ln.pb = ((wave & 1) * 2 + (l8 >> 2)) * 8 + (wave >> 1) * 4 + (l8 & 3);
+  ln.sra = wave * 64 + lane;
+  {
+    const int rho = ln.sra & 127, j = rho >> 4, gg = (rho >> 2) & 3, e = rho & 3;
+    ln.srb = (ln.sra & 128) + (j >> 1) * 32 + gg * 8 + (j & 1) * 4 + e;
+  }
+  // fragment read addresses: lane (g, r) reads chunks 2g and 2g+1 of row (wave row base + 16t + r)
+  v8i fa;
+  {
+    const int m = (ln.r & 7) ^ (ln.r >> 3);
+    const uint32_t lo = (uint32_t)(((2 * ln.g) ^ m) << 4);
+    const uint32_t a0 = lds0 + (uint32_t)(ln.wm0 + ln.r) * 128u + lo;
+    const uint32_t b0 = lds0 + 32768u + (uint32_t)(ln.wn0 + ln.r) * 128u + lo;
+    fa[0] = (int)a0; fa[1] = (int)(a0 ^ 16u); fa[2] = (int)b0; fa[3] = (int)(b0 ^ 16u);
+    fa[4] = (int)(a0 + 65536u); fa[5] = (int)((a0 ^ 16u) + 65536u); fa[6] = (int)(b0 + 65536u); fa[7] = (int)((b0 ^ 16u) + 65536u);
+  }
+  const uint32_t wl = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)wave * 1024u));
+
+  Sched<T, false> sched;
+  sched.init(p);
+  Work w, wnext;
+  bool have = sched.next(p, w, &s_bcast, tid);
+  int first = 1;
+  uint32_t scbuf = 0;
+  const int kh = p.k_iters >> 1;
+  while (have) {
+    // the tile after this one: its first two K steps are requested during this tile's last two.  With
+    // none left the copies read this tile's first steps again; nobody uses them.
+    const bool have_next = sched.next(p, wnext, &s_bcast, tid);
+    if (!have_next) wnext.tc = w.tc;
+    W4TileArgs cur, nxt;
+    w4_tile_args<T>(p, w.tc, ln, cur);
+    w4_tile_args<T>(p, wnext.tc, ln, nxt);
+    v8i sc;
+    sc[0] = (int)(lds0 + 131072u + (uint32_t)(ln.wm0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
+    sc[1] = (int)(lds0 + 131072u + (uint32_t)(256 + ln.wn0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
+    sc[2] = (int)cur.sca; sc[3] = (int)cur.scb; sc[4] = (int)nxt.sca; sc[5] = (int)nxt.scb; sc[6] = 0; sc[7] = 0;
+    if constexpr (T::DT == DT_FP8) {
+      asm volatile(
+#include "w4_kloop_fp8.inc"
+          : [scbuf] "+s"(scbuf)
+          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
+            [A] "s"(cur.A), [B] "s"(cur.B), [An] "s"(nxt.A), [Bn] "s"(nxt.B), [wl] "s"(wl), [kh] "s"(kh), [first] "s"(first)
+          :
+#include "w4_clobbers.inc"
+      );
+    } else {
+      asm volatile(
+#include "w4_kloop_fp4.inc"
+          : [scbuf] "+s"(scbuf)
+          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
+            [A] "s"(cur.A), [B] "s"(cur.B), [An] "s"(nxt.A), [Bn] "s"(nxt.B), [mxa] "s"(cur.mxa), [mxb] "s"(cur.mxb),
+            [mxan] "s"(nxt.mxa), [mxbn] "s"(nxt.mxb), [wl] "s"(wl), [kh] "s"(kh), [first] "s"(first)
+          :
+#include "w4_clobbers.inc"
+      );
+    }
+    if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
+    else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
+    else epilogue_w4<T, DT_F32>(p, w.tc, ln);
+    w.tc = wnext.tc;
+    have = have_next;
+    first = 0;
+  }
+  // the last tile's look-ahead copies still write LDS: they must have landed before the workgroup ends
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (p.mode == MODE_WS && tid == 0) {
+    // the last workgroup to leave rearms the queues for the next launch
+    uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
+    if (done == gridDim.x - 1) {
+      for (int qi = 0; qi <= p.num_xcds * p.counters_per_xcd; ++qi)
+        __hip_atomic_store(p.counters + qi * COUNTER_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+}  // namespace tb

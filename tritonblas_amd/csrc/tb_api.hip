@@ -96,20 +96,22 @@ std::vector<TileInfo> tile_infos(int dt) {
 // taken (measured, 64x64 bf16 tiles: 128x4096x4096 32 -> 22 us, 64x8192x8192 60 -> 39 us with four
 // stages; 2048^3 30 -> 35 us, which the rule avoids).
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast, int64_t total_tiles = 0,
-                            const tb_hw* hw = nullptr) {
+                            const tb_hw* hw = nullptr, bool need_sk = false, int64_t k = 0) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
+  // the hand-scheduled 4-wave kernels run K steps in pairs and have no Stream-K form
+  auto usable = [&](const Variant& x) { return !x.k_step_pairs || (!need_sk && k > 0 && k % (2 * (int64_t)x.bk) == 0); };
   // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
   const char* wenv = getenv("TB_WAVES");
   const int want = wenv ? atoi(wenv) : 0;
   if (want && fast)
     for (int i = 0; i < n; ++i)
-      if (v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
+      if (usable(v[i]) && v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
           (v[i].wm * 10 + v[i].wn == want || v[i].wm * 100 + v[i].wn * 10 + v[i].stages == want))
         return &v[i];
   const Variant* best = nullptr;
   for (int i = 0; i < n; ++i) {
-    if (!(v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk))))
+    if (!(usable(v[i]) && v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && (fast == 0 || (v[i].bm == bm && v[i].bn == bn && v[i].bk == bk))))
       continue;
     if (!best) { best = &v[i]; if (!hw || total_tiles <= 0 || !fast) return best; continue; }   // (listed first: the default depth)
     const int occ = std::max(1, std::min(v[i].minb, hw->lds_bytes / std::max(1, v[i].lds_bytes)));
@@ -231,7 +233,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     int64_t at_once = ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn);
     if (j.schedule == TB_SCHED_STREAMK) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
     if (j.num_groups > 0) at_once = 0;
-    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw);
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw, j.schedule == TB_SCHED_STREAMK && j.num_groups == 0, j.K);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
