@@ -1,0 +1,12 @@
+// The hand-scheduled 4-wave 256x256 kernels (FP8 and MXFP4), see gemm_w4.h.
+#include "gemm_w4.h"
+
+namespace tb {
+
+const void* w4_kernel(int dt) {
+  if (dt == DT_FP8) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP8>>;
+  if (dt == DT_FP4) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP4>>;
+  return nullptr;
+}
+
+}  // namespace tb

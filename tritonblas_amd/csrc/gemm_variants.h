@@ -2,7 +2,6 @@
 #pragma once
 #include <stdint.h>
 #include "gemm_device.h"
-#include "gemm_w4.h"
 
 namespace tb {
 
@@ -22,11 +21,15 @@ constexpr Variant make_variant() {
                  T::FAST ? 1 : 0, T::STAGES, (const void*)&gemm_kernel<T, false>, (const void*)&gemm_kernel<T, true>, 0};
 }
 
-// the hand-scheduled 4-wave kernel of gemm_w4.h for the same tile shape
+// The hand-scheduled 4-wave kernels of gemm_w4.h (256x256 tile, 128-byte K steps) are compiled in a
+// translation unit of their own (gemm_inst_w4.hip), which hands out their addresses.
+const void* w4_kernel(int dt);
+template <int DT>
+using W4Tile = Tile<DT, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>;
 template <class T>
-constexpr Variant make_variant_w4() {
+Variant make_variant_w4() {
   return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, T::LDS_ALLOC, 1,
-                 1, T::STAGES, (const void*)&gemm_kernel_w4<T>, nullptr, 1};
+                 1, T::STAGES, w4_kernel(T::DT), nullptr, 1};
 }
 
 // defined one per translation unit

@@ -21,7 +21,7 @@
 // with no LDS staging -- the LDS already belongs to the next tile's first K steps by then.
 #pragma once
 #include <utility>
-#include "gemm_device.h"
+#include "gemm_variants.h"
 
 namespace tb {
 
@@ -36,6 +36,17 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// A value every lane holds alike, as a scalar register (an "s" operand of an assembly statement must
+// be one; the compiler does not move a value it keeps in a vector register there by itself).
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ uint32_t uniform(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
 // accumulator register a[N] (written by the K loop statement; the compiler never allocates these)
 template <int N>
 __device__ __forceinline__ float acc_read() {
@@ -43,9 +54,6 @@ __device__ __forceinline__ float acc_read() {
   asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
   return x;
 }
-
-template <int DT>
-using W4Tile = Tile<DT, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>;
 
 // what the K loop needs to know about one output tile
 struct W4TileArgs {
@@ -68,8 +76,13 @@ template <class T>
 __device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, W4TileArgs& t) {
   const int rva = tc.m_lim - tc.m0, rvb = tc.n_lim - tc.n0;
   const uint32_t sra = (uint32_t)p.a_sr, srb = (uint32_t)p.b_sr;   // bytes (one-byte storage units)
+#ifdef W4_LAB_SAMETILE
+  t.A = p.A;   // measurement build: every tile reads the operands of tile (0, 0) (all copies hit in L2)
+  t.B = tc.B;
+#else
   t.A = p.A + (int64_t)tc.m0 * p.a_sr;
   t.B = tc.B + (int64_t)tc.n0 * p.b_sr;
+#endif
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     t.off[i] = (int)((uint32_t)min(i * 32 + ln.pa, rva - 1) * sra + ln.c16);
@@ -156,6 +169,55 @@ __device__ __forceinline__ void epilogue_w4(const GemmParams& p, const TileCtx& 
   });
 }
 
+// Fast path of the epilogue: the whole 256x256 tile lies inside C, C rows are 16-byte aligned with
+// unit column stride, 16-bit output, no bias, scale vectors 16-byte aligned.  No per-element bounds
+// handling, and exactly 32 stores per wave, issued as assembly so that the count is known: the next
+// tile's K loop waits for its first copies with "at most N younger memory operations in flight" and
+// has to know how many of those are this epilogue's stores.
+template <class T, int CT, bool NT>
+__device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const TileCtx& tc, const W4Lane& ln) {
+  const int mrow = tc.m0 + ln.wm0 + ln.r;
+  const int ncol = tc.n0 + ln.wn0 + 8 * ln.g;
+  float sav[8];
+  v4f sbv[8];
+  if (p.sa) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sav[i] = p.sa[mrow + i * 16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      sbv[2 * q] = *(const v4f*)(tc.sb + ncol + 32 * q);
+      sbv[2 * q + 1] = *(const v4f*)(tc.sb + ncol + 32 * q + 4);
+    }
+  }
+  uint16_t* c0 = (uint16_t*)p.C + ((int64_t)mrow * p.c_sm + ncol);
+  static_for<8>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    uint16_t* crow = c0 + (int64_t)(i * 16) * p.c_sm;
+    static_for<4>([&](auto Q) {
+      constexpr int q = decltype(Q)::value;
+      float v[8];
+      static_for<8>([&](auto E) {
+        constexpr int e = decltype(E)::value;
+        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3))>();
+      });
+      if (p.sa) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * (sav[i] * sbv[2 * q + (e >> 2)][e & 3]);
+      }
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (CT == DT_F16) h[e] = __builtin_bit_cast(uint16_t, (_Float16)v[e]);
+        else h[e] = __builtin_bit_cast(uint16_t, (__bf16)v[e]);
+      }
+      const v4i pk = {(int)(h[0] | (h[1] << 16)), (int)(h[2] | (h[3] << 16)), (int)(h[4] | (h[5] << 16)), (int)(h[6] | (h[7] << 16))};
+      uint16_t* const dst = crow;   // (assembly operands do not capture: name a local of this lambda)
+      if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off offset:%2 nt" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
+      else asm volatile("global_store_dwordx4 %0, %1, off offset:%2" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
+    });
+  });
+}
+
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
@@ -201,6 +263,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   Work w, wnext;
   bool have = sched.next(p, w, &s_bcast, tid);
   int first = 1;
+  int nst = 0;             // 1: the previous tile's epilogue issued exactly 32 stores per wave (its fast path)
   uint32_t scbuf = 0;
   const int kh = p.k_iters >> 1;
   while (have) {
@@ -215,29 +278,39 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     sc[0] = (int)(lds0 + 131072u + (uint32_t)(ln.wm0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
     sc[1] = (int)(lds0 + 131072u + (uint32_t)(256 + ln.wn0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
     sc[2] = (int)cur.sca; sc[3] = (int)cur.scb; sc[4] = (int)nxt.sca; sc[5] = (int)nxt.scb; sc[6] = 0; sc[7] = 0;
+    const uint8_t *sA = uniform(cur.A), *sB = uniform(cur.B), *sAn = uniform(nxt.A), *sBn = uniform(nxt.B);
+    const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst);
+    scbuf = uniform(scbuf);
     if constexpr (T::DT == DT_FP8) {
       asm volatile(
 #include "w4_kloop_fp8.inc"
           : [scbuf] "+s"(scbuf)
           : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(cur.A), [B] "s"(cur.B), [An] "s"(nxt.A), [Bn] "s"(nxt.B), [wl] "s"(wl), [kh] "s"(kh), [first] "s"(first)
+            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
           :
 #include "w4_clobbers.inc"
       );
     } else {
+      const uint8_t *sMa = uniform(cur.mxa), *sMb = uniform(cur.mxb), *sMan = uniform(nxt.mxa), *sMbn = uniform(nxt.mxb);
       asm volatile(
 #include "w4_kloop_fp4.inc"
           : [scbuf] "+s"(scbuf)
           : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(cur.A), [B] "s"(cur.B), [An] "s"(nxt.A), [Bn] "s"(nxt.B), [mxa] "s"(cur.mxa), [mxb] "s"(cur.mxb),
-            [mxan] "s"(nxt.mxa), [mxbn] "s"(nxt.mxb), [wl] "s"(wl), [kh] "s"(kh), [first] "s"(first)
+            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [mxa] "s"(sMa), [mxb] "s"(sMb),
+            [mxan] "s"(sMan), [mxbn] "s"(sMbn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
           :
 #include "w4_clobbers.inc"
       );
     }
-    if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
+    const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
+                      (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
+    if (fast) {
+      if (p.c_type == DT_BF16) { if (p.c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_BF16, false>(p, w.tc, ln); }
+      else { if (p.c_nt) epilogue_w4_fast<T, DT_F16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_F16, false>(p, w.tc, ln); }
+    } else if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
     else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
     else epilogue_w4<T, DT_F32>(p, w.tc, ln);
+    nst = fast ? 1 : 0;
     w.tc = wnext.tc;
     have = have_next;
     first = 0;

@@ -35,7 +35,7 @@ Register map (VGPR):  0..127  B fragment sets 0/1 (8 fragments x 8 registers eac
                       224..231 inputs: fragment read addresses (A lo, A hi, B lo, B hi) for stage 0, then stage 1
                       232..237 inputs: scale read addresses (A, B), scale copy offsets (A, B) now and next
                       240, 241 scratch: scale read addresses of the current scale buffer
-SGPR 70..81 are scratch (copy cursors, loop counter, scale buffer toggle).
+SGPR 70..82 are scratch (copy cursors, loop counter, scale buffer toggle, first-step flag).
 """
 import sys
 
@@ -43,19 +43,33 @@ STAGE = 65536
 BOFF = 32768
 SC0 = 131072          # scale buffers behind the two stages
 SCBUF = 8192
-BND = 5               # the K-step boundary sits in front of this row block
+NST = 32              # stores per wave of the fast epilogue (256x256 16-bit values, 16 bytes per lane and store)
+import os
+BND = int(os.environ.get("W4GEN_BND", "5"))   # the K-step boundary sits in front of this row block
 
-S_CA, S_CB, S_CSA, S_CSB, S_CNT, S_SCN, S_T, S_SCIN = 70, 72, 74, 76, 78, 79, 80, 81
+S_CA, S_CB, S_CSA, S_CSB, S_CNT, S_SCN, S_T, S_SCIN, S_FIRST = 70, 72, 74, 76, 78, 79, 80, 81, 82
 
 
 class Gen:
-    def __init__(self, fp4, dma_every=1):
+    def __init__(self, fp4, dma_every=1, lab=()):
         self.fp4 = fp4
         self.out = []
         self.nm = 16 if fp4 else 8      # MFMAs per row block
         self.dma_every = dma_every
+        self.lbl = 0
+        # measurement builds (W4GEN_LAB=nomfma,nodma,noread,nobar): leave one kind of instruction out to time
+        # the rest; results are then meaningless
+        self.lab = set(lab)
 
     def e(self, s):
+        if "nomfma" in self.lab and s.startswith("v_mfma"):
+            return
+        if "nodma" in self.lab and s.startswith("global_load_lds"):
+            return
+        if "noread" in self.lab and s.startswith("ds_read"):
+            return
+        if "nobar" in self.lab and s.startswith("s_barrier"):
+            return
         self.out.append(s)
 
     # ---- register names ---------------------------------------------------------------------------
@@ -134,31 +148,77 @@ class Gen:
                 f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
 
     # ---- one K step -------------------------------------------------------------------------------
-    def step(self, p, nxt, prefetch, last_iter_even=False):
-        """K step in stage p (= B set p, scale set p).  nxt: the copies issued behind the boundary read
-        the next tile.  prefetch: request the following step's fragments in the tail."""
+    def wait_vm(self, n, n_stores, n_cons):
+        """s_waitcnt vmcnt(n) in the steady state.  While s82 is set (first K steps of a tile) the previous
+        tile's epilogue stores are younger than the copies waited for: with %[nst] they are exactly 32 per
+        wave and the wait allows for them (n_stores), otherwise it assumes none (n_cons)."""
+        self.lbl += 1
+        f, g, d = (f"W4_V{x}{self.lbl}_%=" for x in "FGD")
+        return [f"s_cmp_lg_u32 s{S_FIRST}, 0", f"s_cbranch_scc1 {f}", f"s_waitcnt vmcnt({n})", f"s_branch {d}",
+                f"{f}:", "s_cmp_lg_u32 %[nst], 0", f"s_cbranch_scc1 {g}", f"s_waitcnt vmcnt({n_cons})", f"s_branch {d}",
+                f"{g}:", f"s_waitcnt vmcnt({n_stores})", f"{d}:"]
+
+    def step(self, p, nxt, prefetch):
+        """K step in stage p (= B set p, scale set p).  nxt: the copies issued in this step read the
+        next tile.  prefetch: request the following step's fragments in the tail.
+
+        Two sync points (wait + s_barrier) per step, each followed by copies of step +2 into LDS that
+        every wave has just declared free:
+          X, in front of row block 1: this step's B fragments and A fragments 0..3 are in registers
+             -> B half of the stage and the A rows of row blocks 0..3 ("A lo") take step +2;
+             it also publishes "A hi" of THIS step (row blocks 4..7), which is read from here on;
+          Y, in front of row block 5 (the step boundary): A fragments 4..7 are in registers
+             -> "A hi" takes step +2; it publishes B and "A lo" of the NEXT step for the tail's reads.
+        Every copy is therefore waited for one and a half K steps after it was issued, and two to
+        three bursts overlap in time: one burst per step that has to land within one step leaves the
+        L2 -> LDS path idle for the latency of its first byte and then stalls the MFMAs at the wait.
+        vmcnt counts in issue order, so each wait names how many younger copies may stay in flight."""
         nm = self.nm
+        total = 8 * nm
         self.e(f"; ---- K step, stage {p}{' (copies: next tile)' if nxt else ''}{'' if prefetch else ' (last of the tile)'}")
-        for i in range(BND):
-            if i + 3 <= 7:
-                for l in self.frag_read(self.vA(i + 3), 0, p, i + 3):
-                    self.e(l)
-            self.e("s_waitcnt lgkmcnt(6)" if i + 3 <= 7 else "s_waitcnt lgkmcnt(0)")
-            for s in range(nm):
-                self.e(self.mfma(p, i, s))
-        # boundary: every LDS read of this step has returned, the next step's copies have landed,
-        # and every wave says so; then the freed stage takes the copies of step +2
-        self.e("s_waitcnt lgkmcnt(0)")
-        self.e("s_waitcnt vmcnt(0)")
-        self.e("s_barrier")
-        tail = 3 * nm
-        extras = [[] for _ in range(tail)]
+        pre = [[] for _ in range(total)]      # in front of MFMA slot m
+        post = [[] for _ in range(total)]     # behind it
+        ops = self.dma(p, nxt)
+        lo = [ops[i] for i in (0, 1, 4, 5)]                 # A rows of row blocks 0..3 (both wave rows)
+        hi = [ops[i] for i in (2, 3, 6, 7)]
+        ops_b = ops[8:]
+        adv = self.dma_advance()
+        adv_a, adv_b = adv[:2], adv[2:]
+        sc = self.scale_dma(nxt) if (self.fp4 and p == 0) else []
+        nx = len(ops_b) + len(lo) + len(sc)                # copies issued behind X of this step
+        nx_other = 12 + (2 if (self.fp4 and p == 1) else 0)   # ... behind X of the neighbouring steps
+        # row block 0
+        pre[0] += self.frag_read(self.vA(3), 0, p, 3)
+        pre[0].append("s_waitcnt lgkmcnt(6)")
+        # X
+        # (X of step 0: nothing of this tile may be assumed younger than the stores; X of step 1: the
+        # steady-state count already demands that the stores are done)
+        pre[nm] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx_other + 4, nx_other + 4 + NST, 0 if p == 0 else nx_other + 4) + ["s_barrier"]
+        if p == 1:
+            post[nm].append(f"s_mov_b32 s{S_FIRST}, 0")
+        pre[nm] += self.frag_read(self.vA(4), 0, p, 4)
+        xops = ops_b + lo + sc
+        span = 4 * nm - 2
+        for n, op in enumerate(xops):
+            post[nm + n * span // len(xops)] += op
+        post[5 * nm - 2] += adv_b
+        pre[2 * nm] += self.frag_read(self.vA(5), 0, p, 5)
+        pre[3 * nm] += self.frag_read(self.vA(6), 0, p, 6)
+        pre[4 * nm] += self.frag_read(self.vA(7), 0, p, 7)
+        pre[4 * nm].append("s_waitcnt lgkmcnt(6)")
+        # Y
+        tail0 = BND * nm
+        if p == 0:
+            pre[tail0] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx + 4, nx + 4 + NST, nx) + ["s_barrier"]
+        else:
+            pre[tail0] += ["s_waitcnt lgkmcnt(0)", f"s_waitcnt vmcnt({nx + 4})", "s_barrier"]
+        tail = total - tail0
         q = p ^ 1
         if prefetch:
             lds = []
             if self.fp4 and p == 1:
                 # the next step opens a new scale group: it sits in the other buffer
-                extras[0] += [f"v_xor_b32 v240, {SCBUF}, v240", f"v_xor_b32 v241, {SCBUF}, v241"]
+                post[tail0] += [f"v_xor_b32 v240, {SCBUF}, v240", f"v_xor_b32 v241, {SCBUF}, v241"]
             for j in range(8):
                 lds += self.frag_read(self.vB(q, j), 1, q, j)
             if self.fp4:
@@ -166,21 +226,17 @@ class Gen:
             lds += self.frag_read(self.vA(0), 0, q, 0)
             span = tail // 2
             for n, l in enumerate(lds):
-                extras[n * span // len(lds)].append(l)
-            extras[tail // 2] += self.frag_read(self.vA(1), 0, q, 1)
-            extras[tail * 5 // 6] += self.frag_read(self.vA(2), 0, q, 2)
-        ops = self.dma(p, nxt)
-        for n, op in enumerate(ops):
-            extras[min(n * self.dma_every, tail - 2)] += op
-        pos = min(len(ops) * self.dma_every, tail - 2)
-        extras[pos] += self.dma_advance()
-        if self.fp4 and p == 0:
-            for op in self.scale_dma(nxt):
-                extras[min(pos + 1, tail - 1)] += op
-        for m in range(tail):
-            i, s = BND + m // nm, m % nm
-            self.e(self.mfma(p, i, s))
-            for l in extras[m]:
+                post[tail0 + n * span // len(lds)].append(l)
+            post[tail0 + tail // 2] += self.frag_read(self.vA(1), 0, q, 1)
+            post[tail0 + tail * 5 // 6] += self.frag_read(self.vA(2), 0, q, 2)
+        for n, op in enumerate(hi):
+            post[tail0 + n * (tail - 2) // len(hi)] += op
+        post[total - 2] += adv_a
+        for m in range(total):
+            for l in pre[m]:
+                self.e(l)
+            self.e(self.mfma(p, m // nm, m % nm))
+            for l in post[m]:
                 self.e(l)
 
     # ---- the whole K loop of one tile -------------------------------------------------------------------
@@ -203,8 +259,9 @@ class Gen:
                 for l in op:
                     e(l)
         for st in (0, 1):
-            for op in self.dma(st, False):
-                for l in op:
+            ops = self.dma(st, False)
+            for n in (8, 9, 10, 11, 12, 13, 14, 15, 0, 1, 4, 5, 2, 3, 6, 7):   # B, A lo, A hi: the order the steps use
+                for l in ops[n]:
                     e(l)
             for l in self.dma_advance():
                 e(l)
@@ -224,6 +281,7 @@ class Gen:
             e(f"s_addc_u32 s{S_CSB + 1}, s{S_CSB + 1}, 0")
             e(f"s_xor_b32 s{S_SCN}, s{S_SCN}, {SCBUF}")
         e("W4_ENTRY%=:")
+        e(f"s_mov_b32 s{S_FIRST}, 1")
         # (either way s79 now names the buffer the NEXT scale group goes to)
         if fp4:
             e(f"v_add_u32 v240, s{S_SCIN}, v232")
@@ -270,7 +328,7 @@ class Gen:
 
 
 def clobbers():
-    names = [f"v{i}" for i in range(192)] + ["v240", "v241"] + [f"a{i}" for i in range(256)] + [f"s{i}" for i in range(70, 82)]
+    names = [f"v{i}" for i in range(192)] + ["v240", "v241"] + [f"a{i}" for i in range(256)] + [f"s{i}" for i in range(70, 83)]
     names += ["memory", "vcc", "scc", "m0"]
     lines = []
     for i in range(0, len(names), 16):
@@ -283,8 +341,9 @@ def main():
     if what == "clobbers":
         sys.stdout.write(clobbers())
         return
-    every = int(sys.argv[2]) if len(sys.argv) > 2 else (1 if what == "fp8" else 2)
-    g = Gen(what == "fp4", every)
+    import os
+    every = int(os.environ.get("W4GEN_DMA_EVERY", "1" if what == "fp8" else "2"))
+    g = Gen(what == "fp4", every, [x for x in os.environ.get("W4GEN_LAB", "").split(",") if x])
     g.kloop()
     sys.stdout.write(g.text())
 
