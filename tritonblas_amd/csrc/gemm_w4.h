@@ -212,6 +212,9 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
       }
       const v4i pk = {(int)(h[0] | (h[1] << 16)), (int)(h[2] | (h[3] << 16)), (int)(h[4] | (h[5] << 16)), (int)(h[6] | (h[7] << 16))};
       uint16_t* const dst = crow;   // (assembly operands do not capture: name a local of this lambda)
+#ifdef W4_LAB_NOSTORE
+      if (p.debug == 12345)         // measurement build: no stores (the condition keeps the code alive)
+#endif
       if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off offset:%2 nt" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
       else asm volatile("global_store_dwordx4 %0, %1, off offset:%2" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
     });
@@ -260,6 +263,13 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
 
   Sched<T, false> sched;
   sched.init(p);
+#ifdef W4_LAB_STAGGER
+  {
+    // measurement build: delay the start of workgroups by (id / div) % mod microseconds (debug = div*1000 + mod*... )
+    const int unit = p.debug / 10000, div = (p.debug / 100) % 100, mod = p.debug % 100;
+    if (mod > 0) { const int n = ((int)blockIdx.x / max(div, 1)) % mod * unit; for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(32); }
+  }
+#endif
   Work w, wnext;
   bool have = sched.next(p, w, &s_bcast, tid);
   int first = 1;
@@ -304,9 +314,18 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     }
     const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
                       (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
+    // Every workgroup reaches its epilogue at about the same time, so C arrives as bursts of 32 MB; the
+    // L2s take such a burst as ordinary write-back lines and drain it behind the next K steps, while
+    // non-temporal stores go to the fabric at once and hold the waves at the store queue (measured:
+    // FP8 8192x28672x8192 1.24 -> 1.20 ms, MXFP4 8192x8192x16384 0.440 -> 0.415 ms without the hint).
+#ifdef W4_LAB_NT
+    const bool c_nt = p.c_nt;
+#else
+    const bool c_nt = false;
+#endif
     if (fast) {
-      if (p.c_type == DT_BF16) { if (p.c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_BF16, false>(p, w.tc, ln); }
-      else { if (p.c_nt) epilogue_w4_fast<T, DT_F16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_F16, false>(p, w.tc, ln); }
+      if (p.c_type == DT_BF16) { if (c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_BF16, false>(p, w.tc, ln); }
+      else { if (c_nt) epilogue_w4_fast<T, DT_F16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_F16, false>(p, w.tc, ln); }
     } else if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
     else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
     else epilogue_w4<T, DT_F32>(p, w.tc, ln);

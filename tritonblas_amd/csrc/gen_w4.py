@@ -70,6 +70,12 @@ class Gen:
             return
         if "nobar" in self.lab and s.startswith("s_barrier"):
             return
+        if "novm" in self.lab and s.startswith("s_waitcnt vmcnt"):
+            return
+        if "nolgk0" in self.lab and s == "s_waitcnt lgkmcnt(0)":
+            return
+        if "nolgk" in self.lab and s.startswith("s_waitcnt lgkmcnt"):
+            return
         self.out.append(s)
 
     # ---- register names ---------------------------------------------------------------------------
