@@ -45,6 +45,9 @@ enum {
   TB_I8 = 5         /* operands (int32 sums, persistent_gemm.py:75); as output only with TB_I8 operands: fp32 epilogue
                        result truncated toward zero and saturated to [-128, 127]                    */
 };
+/* TB_FP8_E4M3 is also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 operands: the fp32 epilogue
+ * result is clamped to +-448 and rounded to nearest even (the reference's a8w8 oracle,
+ * tests/test_matmul_a8w8_lt.py:11-38). */
 
 /* ---- schedules ------------------------------------------------------------------------------ */
 enum {
@@ -132,9 +135,15 @@ typedef struct tb_gemm_desc {
   int32_t grid;               /* workgroups to launch; 0 = default (what is co-resident).  A Stream-K
                                  grid beyond what is co-resident is replaced by the default          */
   int32_t counters_per_xcd;
-  void* workspace;            /* tb_workspace_bytes() bytes, zero-initialised once by the caller     */
+  void* workspace;            /* tb_workspace_bytes() bytes, 256-byte aligned, zero-initialised once by
+                                 the caller.  One workspace serves Stream-K and work-stealing launches in
+                                 any order (their regions are disjoint, see tb_workspace_layout)          */
   size_t workspace_bytes;
-  uint32_t epoch;             /* Stream-K: must differ from the previous launch on this workspace    */
+  uint32_t epoch;             /* Stream-K: tags this launch's partial tiles.  Never 0 (a launch that needs
+                                 the workspace is refused with TB_ERR_BAD_ARGUMENT), and never a value an
+                                 earlier launch on this workspace used since it was last zeroed: count
+                                 upwards (flags are not cleared between launches, a stale flag of an equal
+                                 epoch would pass for published)                                          */
   uint32_t spin_limit;        /* Stream-K: bound on flag polls per wait; 0 = default                 */
   /* work stealing only (config.py:23, persistent_gemm_work_stealing.py:70-81): */
   const int32_t* cu_mask;     /* device int32[cu_mask_len] or NULL; workgroup i leaves at once when
@@ -159,6 +168,14 @@ int tb_gemm(const tb_gemm_desc* desc, void* stream);
 
 /* Bytes of workspace tb_gemm needs for this descriptor (0 for the persistent schedule). */
 size_t tb_workspace_bytes(const tb_gemm_desc* desc);
+
+/* Byte offsets of the regions of a workspace: [0, 256) control words -- word 0 is the status (set to 1
+ * when a Stream-K wait ran into spin_limit: the tile concerned was then stored as NaN; cleared only by the
+ * caller), word 1 counts finished work-stealing workgroups; *counters_offset: work-stealing queue
+ * counters, one per 256-byte line; *flags_offset: Stream-K flags (one word per workgroup), the partial
+ * tiles follow at the next 256-byte boundary behind `grid` flags.  Replaces the separate buffers of
+ * matmul_preamble (config.py:86-134). */
+int tb_workspace_layout(size_t* counters_offset, size_t* flags_offset);
 
 /* ---- MXFP4 GEMM (replaces matmul_fp4, matmul.py:519-625) ------------------------------------- */
 typedef struct tb_gemm_fp4_desc {
@@ -246,6 +263,13 @@ int tb_ws_queue_tile(int32_t ws_mode, int32_t queue, int32_t idx, int32_t total_
                      int32_t counters_per_xcd, int32_t local_tiles_per_xcd, int32_t* count, int32_t* tile);
 
 /* ---- misc ----------------------------------------------------------------------------------- */
+/* Tuning and test hooks.  Each has an environment variable that is read once, when the library first
+ * plans a launch (TB_WAVES, TB_NO_MXLDS, TB_NO_CLINE, TB_NO_SKINNY, TB_SKINNY, TB_GRID, TB_PANEL,
+ * TB_NO_COLUMN_SPLIT, TB_FORCE_COLUMN_SPLIT, TB_QUANT_DIV64); this call changes one afterwards, by its lower-case name
+ * without the prefix ("waves", "no_skinny", ...; "panel" -1 = the library's choice).  Process-wide; not
+ * meant for production callers.  No counterpart in the reference. */
+int tb_debug_option(const char* name, int value);
+
 const char* tb_status_string(int status);
 int tb_abi_version(void);
 

@@ -16,11 +16,19 @@ import torch
 from . import mxfp4
 
 
+def _div_by_scalar_as_on_gpu(t: torch.Tensor, s: float) -> torch.Tensor:
+    """``tensor / python_scalar`` as torch evaluates it on a GPU: one multiplication by the scalar's fp32
+    reciprocal (its element-wise kernels fold the division), which differs from a true division by one
+    unit in the last place for some inputs.  The reference's quantisation recipe only ever runs on the
+    GPU, so this -- not CPU torch's true division -- is the arithmetic behind its scales."""
+    return t * torch.tensor(1.0 / s, dtype=torch.float32)
+
+
 def quantize_per_channel_fp8(x: torch.Tensor, axis: int, dtype=torch.float8_e4m3fn, min_scale: float = 1e-8):
     """include/tritonblas/utils.py:340-377: amax -> scale = amax/448 -> q = (x * (1/scale)).to(fp8)."""
     base = x.to(torch.float32)
     max_abs = torch.clamp(base.abs().amax(dim=axis, keepdim=True), min=min_scale)
-    scale = max_abs / torch.finfo(dtype).max
+    scale = _div_by_scalar_as_on_gpu(max_abs, torch.finfo(dtype).max)
     inv = 1.0 / scale
     q = (base * inv).to(dtype)
     return q, scale.squeeze(axis).to(torch.float32)
@@ -31,7 +39,7 @@ def quantize_per_channel_int8(x: torch.Tensor, axis: int, min_scale: float = 1e-
     q = clamp(round(x * (1/scale)), -127, 127).to(int8)."""
     base = x.to(torch.float32)
     max_abs = torch.clamp(base.abs().amax(dim=axis, keepdim=True), min=min_scale)
-    scale = max_abs / 127.0
+    scale = _div_by_scalar_as_on_gpu(max_abs, 127.0)
     q = torch.round(base * (1.0 / scale)).clamp_(-127.0, 127.0).to(torch.int8)
     return q, scale.squeeze(axis).to(torch.float32)
 

@@ -80,13 +80,13 @@ def test_every_16bit_tile_variant(m, n, k, dtype, tile):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
 @pytest.mark.parametrize("stages", [3, 4])
 @pytest.mark.parametrize("m,n,k", [(128, 512, 4096), (300, 200, 2304), (64, 64, 128), (512, 1024, 640)])
-def test_deep_pipeline_variants_of_the_small_tile(dtype, stages, m, n, k, monkeypatch):
+def test_deep_pipeline_variants_of_the_small_tile(dtype, stages, m, n, k, tb_option):
     """The 64x64 tile exists with 2, 3 and 4 copy stages; the library takes a deeper one while all tiles
-    are resident at once.  Here every depth is forced (TB_WAVES = waves_m, waves_n, stages), K both
+    are resident at once.  Here every depth is forced (hook "waves" = waves_m, waves_n, stages), K both
     shorter and longer than the pipeline, ragged edges, Stream-K on top."""
     import tritonblas_amd as tb
-    monkeypatch.setenv("TB_WAVES", f"22{stages}")
-    monkeypatch.setenv("TB_NO_SKINNY", "1")
+    tb_option("waves", 220 + stages)
+    tb_option("no_skinny", 1)
     _say(f"deep pipeline {dtype} stages={stages} {m}x{n}x{k}")
     quant = dtype == torch.float8_e4m3fn
     if quant:
@@ -346,12 +346,12 @@ def test_streamk_workspace_reuse_with_new_data(m, n, k, grid):
 
 
 @pytest.mark.parametrize("kernel", ["streaming", "streamk"])
-def test_decode_shape_small(kernel, monkeypatch):
+def test_decode_shape_small(kernel, tb_option):
     """The decode configuration's shape class (tiny M, long K) at a size the oracle finishes quickly:
     through the streaming skinny-M kernel and through the tile kernel's Stream-K fixup (the library
-    picks between them by model time; TB_SKINNY / TB_NO_SKINNY force the choice)."""
+    picks between them by model time; the hooks "skinny" / "no_skinny" force the choice)."""
     import tritonblas_amd as tb
-    monkeypatch.setenv("TB_NO_SKINNY" if kernel == "streamk" else "TB_SKINNY", "1")
+    tb_option("no_skinny" if kernel == "streamk" else "skinny", 1)
     m, n, k = 32, 1024, 7168
     aq, bq, sa, sb = _a8w8_case(m, n, k, seed=21)
     a, b = aq.cuda(), bq.T.contiguous().cuda().T
@@ -368,13 +368,13 @@ def test_decode_shape_small(kernel, monkeypatch):
                          [(m, 24576 + 40, 256) for m in (7, 32, 64)])   # wide N: 64-column workgroups
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
 @pytest.mark.parametrize("forced", [True, False])
-def test_skinny_rows(m, n, k, dtype, forced, monkeypatch):
+def test_skinny_rows(m, n, k, dtype, forced, tb_option):
     """Every row-block count of the streaming kernel and both column widths of its workgroups, ragged N,
     bias, all three element types; once forced onto the streaming kernel, once with the library's own
     choice between it and the tile kernels."""
     import tritonblas_amd as tb
     if forced:
-        monkeypatch.setenv("TB_SKINNY", "1")
+        tb_option("skinny", 1)
     _say(f"skinny {m}x{n}x{k} {dtype} forced={forced}")
     if dtype == torch.float8_e4m3fn:
         aq, bq, sa, sb = _a8w8_case(m, n, k, seed=31)
@@ -608,7 +608,7 @@ def test_fp4_fast_kernels_random_scales(tile, m, n, k):
 # ---- column split of a partial last round -----------------------------------------------------------
 @pytest.mark.parametrize("kind", ["fp8", "bf16", "bias"])
 @pytest.mark.parametrize("shape", [(2048, 28672, 512), (1536, 14336 + 40, 256), (1100, 20000, 384)])
-def test_column_split(kind, shape, monkeypatch):
+def test_column_split(kind, shape, tb_option):
     """More tiles than the resident grid holds and a partial last round: the library may run the columns
     that fill whole rounds with the selected tile and the rest as a second launch with another tile.
     Forced here; every element of C must equal the one-launch result bit for bit (each output element
@@ -622,9 +622,9 @@ def test_column_split(kind, shape, monkeypatch):
     w = torch.randn(n, k, generator=g).bfloat16()
     bias = torch.randn(n, generator=g).bfloat16() if kind == "bias" else None
     outs = {}
-    for name, env in (("one", {"TB_NO_COLUMN_SPLIT": "1", "TB_FORCE_COLUMN_SPLIT": "0"}), ("split", {"TB_NO_COLUMN_SPLIT": "0", "TB_FORCE_COLUMN_SPLIT": "1"})):
+    for name, env in (("one", {"no_column_split": 1, "force_column_split": 0}), ("split", {"no_column_split": 0, "force_column_split": 1})):
         for key, val in env.items():
-            monkeypatch.setenv(key, val)
+            tb_option(key, val)
         c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         # the tall tile named outright, so that the tile count (and with it the seam) is known
         import types

@@ -43,14 +43,14 @@ def test_random(shape, dtype, hadamard):
 @pytest.mark.parametrize("hadamard", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(1, 32), (3, 64), (257, 4096), (1000, 96), (37, 14336)])
-def test_both_index_paths(shape, dtype, hadamard, monkeypatch):
+def test_both_index_paths(shape, dtype, hadamard, tb_option):
     """Below 2^31 items the kernel splits an item index into (row, column) with a multiply-high by a
     reciprocal the host computes; the kernel for larger tensors divides.  Both are forced here on row
     lengths that are and are not powers of two, and must give the oracle's bytes."""
     g = torch.Generator().manual_seed(11)
     x = torch.randn(shape, generator=g).to(dtype)
-    for div64 in ("0", "1"):
-        monkeypatch.setenv("TB_QUANT_DIV64", div64)
+    for div64 in (0, 1):
+        tb_option("quant_div64", div64)
         _assert_same(x, hadamard)
 
 

@@ -1,0 +1,241 @@
+"""GPU tests of the hand-scheduled 4-wave 256x256 kernels (FP8 and MXFP4) and of the workspace rules.
+
+The 4-wave kernels form every sum in the same order as the 8-wave kernels of the same tile (same MFMA
+instruction, same K grouping), so the two must agree bit for bit; the 8-wave kernels are checked against
+the CPU oracle throughout tests/test_gemm_gpu.py, and the cases here check the 4-wave ones against the
+oracle as well.  All launches go through the C ABI."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as OG
+from oracle import mxfp4 as OM
+
+pytestmark = pytest.mark.gpu
+TOL_Q = 1e-2
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _fp8_case(m, n, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(n, k, generator=torch.Generator().manual_seed(seed + 10000)).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    bq, sb = OG.quantize_per_channel_fp8(w.T, axis=0)
+    return aq, bq, sa, sb
+
+
+def _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=torch.bfloat16, bias=None, work_stealing=False):
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import persistent_matmul_lt
+    m, k = aq.shape
+    n = bq.shape[1]
+    tb_option("waves", waves)
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, out_dtype, a.device)
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 128
+    c = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+    cfg = tb.matmul_preamble(sel) if work_stealing else None
+    persistent_matmul_lt(a, b, c, sel, cfg, bias=None if bias is None else bias.cuda(), a_scale=sa.cuda(), b_scale=sb.cuda(),
+                         quantized=True, work_stealing=work_stealing)
+    return c.cpu()
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (256, 256, 2048), (512, 768, 512), (300, 500, 768), (1, 257, 256),
+                                   (1024, 2048, 1024), (2560, 2304, 512)])
+def test_fp8_four_wave_kernel(m, n, k, tb_option):
+    """Whole and ragged tiles, one to many tiles per workgroup (2560x2304 = 90 tiles): oracle parity and
+    bit-equality with the 8-wave kernel."""
+    _say(f"w4 fp8 {m}x{n}x{k}")
+    aq, bq, sa, sb = _fp8_case(m, n, k, 71)
+    new = _run_fp8(aq, bq, sa, sb, 22, tb_option)
+    old = _run_fp8(aq, bq, sa, sb, 24, tb_option)
+    want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
+    assert OG.rel_fro_error(new.float(), want.float()) <= TOL_Q
+    assert torch.equal(new.view(torch.int16), old.view(torch.int16))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_fp8_four_wave_epilogue_variants(out_dtype, with_bias, tb_option):
+    """fp16 / fp32 output and a per-column bias take the general epilogue of the 4-wave kernel."""
+    m, n, k = 384, 640, 512
+    aq, bq, sa, sb = _fp8_case(m, n, k, 72)
+    bias = torch.randn(n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16) if with_bias else None
+    new = _run_fp8(aq, bq, sa, sb, 22, tb_option, out_dtype=out_dtype, bias=bias)
+    old = _run_fp8(aq, bq, sa, sb, 24, tb_option, out_dtype=out_dtype, bias=bias)
+    want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb)
+    if with_bias:
+        want = want + bias.float()[None, :]
+    assert OG.rel_fro_error(new.float(), want.to(out_dtype).float()) <= TOL_Q
+    assert torch.equal(new, old)
+
+
+def test_fp8_four_wave_work_stealing(tb_option):
+    """The 4-wave kernel under the work-stealing schedule (tiles from the atomic queues, one tile looked
+    ahead): bit-identical to its data-parallel result, three launches on one config without a reset."""
+    m, n, k = 1536, 2304, 512
+    aq, bq, sa, sb = _fp8_case(m, n, k, 73)
+    static = _run_fp8(aq, bq, sa, sb, 22, tb_option)
+    for rep in range(3):
+        ws = _run_fp8(aq, bq, sa, sb, 22, tb_option, work_stealing=True)
+        assert torch.equal(static.view(torch.int16), ws.view(torch.int16)), f"launch {rep}"
+
+
+def test_fp8_four_wave_needs_an_even_number_of_k_steps(tb_option):
+    """K = 3 steps of 128: the library must fall back to the 8-wave kernel by itself and stay correct."""
+    m, n, k = 512, 512, 384
+    aq, bq, sa, sb = _fp8_case(m, n, k, 74)
+    got = _run_fp8(aq, bq, sa, sb, 0, tb_option)
+    want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
+    assert OG.rel_fro_error(got.float(), want.float()) <= TOL_Q
+
+
+def _fp4_case(m, n, k, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.standard_normal((n, k)).astype(np.float32)
+    xq, xs = OM.mxfp4_quant(x)
+    wq, ws = OM.mxfp4_quant(w)
+    return torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs), torch.from_numpy(ws)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (256, 256, 4096), (512, 768, 1024), (300, 500, 1536), (2048, 1280, 2048)])
+def test_fp4_four_wave_kernel(m, n, k, tb_option):
+    import tritonblas_amd as tb
+    _say(f"w4 fp4 {m}x{n}x{k}")
+    xq, wq, xs, ws = _fp4_case(m, n, k, 75)
+    # scale bytes far from 127 in some blocks: the E8M0 operands of the scaled MFMA must be honoured
+    xs[::3, ::2] = 120
+    ws[1::4, 1::3] = 133
+    outs = {}
+    for waves in (22, 24):
+        tb_option("waves", waves)
+        c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        tb.matmul_fp4(xq.cuda(), wq.cuda(), c, xs.cuda(), ws.cuda(), block_m=256, block_n=256, block_k=256)
+        outs[waves] = c.cpu()
+    want = OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True).to(torch.bfloat16)
+    assert OG.rel_fro_error(outs[22].float(), want.float()) <= TOL_Q
+    assert torch.equal(outs[22].view(torch.int16), outs[24].view(torch.int16))
+
+
+# ---- workspace rules --------------------------------------------------------------------------------------
+def test_streamk_then_work_stealing_on_one_config():
+    """Stream-K flags and work-stealing counters live in disjoint regions of the workspace: a Stream-K
+    launch whose workgroups 64, 128, 192 publish (explicit grid) followed by work stealing on the SAME
+    config, and the other way round, both against the oracle."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    dtype = torch.bfloat16
+    m = n = k = 2048
+    g = torch.Generator().manual_seed(81)
+    a_cpu, b_cpu = (torch.randn(m, k, generator=g) * 0.5).to(dtype), (torch.randn(k, n, generator=g) * 0.5).to(dtype)
+    want = OG.ref_gemm(a_cpu, b_cpu, torch.float32).to(dtype)
+    a, b = a_cpu.cuda(), b_cpu.cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device, streamk=True)
+    cfg = tb.matmul_preamble(sel)
+    for order in (("sk", "ws", "sk", "ws"), ("ws", "sk", "ws")):
+        cfg.reset(streamk=True, work_stealing=True)
+        for what in order:
+            c = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+            if what == "sk":
+                streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=200)
+            else:
+                tb.matmul_lt(a, b, c, sel, cfg, work_stealing=True)
+            err = OG.rel_fro_error(c.float().cpu(), want.float())
+            assert err <= 1e-3, f"{order} at {what}: {err}"
+        assert cfg.status() == 0
+
+
+def test_streamk_epoch_zero_is_refused():
+    """A zero-initialised descriptor (epoch 0) on a zeroed workspace would match every flag at once."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    m, n, k = 256, 256, 4096
+    a = torch.randn(m, k, device="cuda").half()
+    b = torch.randn(k, n, device="cuda").half()
+    c = torch.zeros(m, n, device="cuda").half()
+    d = _lib.tb_gemm_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+    d.a_type = d.b_type = d.c_type = _lib.TB_F16
+    d.m, d.n, d.k = m, n, k
+    d.a_stride_m, d.a_stride_k = a.stride()
+    d.b_stride_k, d.b_stride_n = b.stride()
+    d.c_stride_m, d.c_stride_n = c.stride()
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.schedule, d.grid = _lib.TB_SCHED_STREAMK, 64
+    need = lib.tb_workspace_bytes(d)
+    assert need > 0
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    d.workspace, d.workspace_bytes = ws.data_ptr(), need
+    d.epoch = 0
+    assert lib.tb_gemm(d, _lib.stream_handle()) == _lib.TB_ERR_BAD_ARGUMENT
+    d.epoch = 1
+    assert lib.tb_gemm(d, _lib.stream_handle()) == _lib.TB_OK
+    torch.cuda.synchronize()
+    assert OG.rel_fro_error(c.float().cpu(), (a.float().cpu() @ b.float().cpu()).half().float()) <= 1e-3
+
+
+def test_streamk_poll_bound_poisons_the_tile():
+    """With a poll bound of one, owners give up before their partners publish (every kernel still ends
+    normally): the tiles they could not finish must hold NaN, never stale memory, the status word must be
+    set and MatmulConfig.check() must raise.  A later launch with the default bound is correct again."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    dtype = torch.bfloat16
+    m, n, k = 256, 256, 16384
+    g = torch.Generator().manual_seed(82)
+    a_cpu, b_cpu = (torch.randn(m, k, generator=g) * 0.5).to(dtype), (torch.randn(k, n, generator=g) * 0.5).to(dtype)
+    want = OG.ref_gemm(a_cpu, b_cpu, torch.float32).to(dtype)
+    a, b = a_cpu.cuda(), b_cpu.cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device, streamk=True)
+    cfg = tb.matmul_preamble(sel)
+    cfg.spin_limit = 1
+    c = torch.full((m, n), 7.0, dtype=dtype, device="cuda")
+    streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=256)
+    torch.cuda.synchronize()
+    got = c.float().cpu()
+    if cfg.status() != 0:
+        assert torch.isnan(got).any()
+        ok = ~torch.isnan(got)
+        assert torch.equal(got[ok], want.float()[ok]) or OG.rel_fro_error(got[ok], want.float()[ok]) <= 1e-3
+        with pytest.raises(RuntimeError):
+            cfg.check()
+        assert cfg.status() == 0
+    else:   # every partner happened to be early: then the result must simply be right
+        assert OG.rel_fro_error(got, want.float()) <= 1e-3
+    cfg.spin_limit = 0
+    c2 = torch.zeros(m, n, dtype=dtype, device="cuda")
+    streamk_matmul_lt(a, b, c2, sel, cfg, sk_grid=256)
+    assert OG.rel_fro_error(c2.float().cpu(), want.float()) <= 1e-3
+    cfg.check()
+
+
+# ---- e4m3 output ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (100, 300, 640), (512, 1024, 512)])
+@pytest.mark.parametrize("streamk", [False, True])
+def test_a8w8_fp8_output(m, n, k, streamk):
+    """a8w8 with an e4m3 result: clamp to +-448, round to nearest even -- the reference's oracle and
+    tolerances for this case (tests/test_matmul_a8w8_lt.py:11-38, :108-112: atol 2.0, rtol 0.2)."""
+    import tritonblas_amd as tb
+    aq, bq, sa, sb = _fp8_case(m, n, k, 91)
+    sa = sa * 40.0   # push part of the result beyond the e4m3 range so that the clamp is exercised
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    c = torch.zeros(m, n, dtype=torch.float8_e4m3fn, device="cuda")
+    tb.matmul_a8w8(a, b, sa.cuda(), sb.cuda(), c, enable_streamk=streamk)
+    want = OG.ref_gemm(aq, bq, torch.float8_e4m3fn, a_scale=sa, b_scale=sb)
+    got = c.float().cpu()
+    assert not torch.isnan(got).any()
+    assert got.abs().max() <= 448.0
+    torch.testing.assert_close(got, want.float(), atol=2.0, rtol=0.2)
+    # the rounding itself: at most one e4m3 step away from the oracle's cast, and mostly identical
+    same = (c.cpu().view(torch.uint8) == want.view(torch.uint8)).float().mean().item()
+    assert same >= 0.99, f"only {same:.4f} of the e4m3 codes match the oracle's"

@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
     "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile", "tb_hierarchical_split",
+    "tb_workspace_layout", "tb_debug_option",
 ]
 
 
@@ -118,10 +119,24 @@ def load():
     lib.tb_default_panel.argtypes = [C.c_int32] * 3
     lib.tb_ws_queue_tile.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32)] * 2
     lib.tb_hierarchical_split.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    lib.tb_workspace_layout.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    lib.tb_debug_option.argtypes = [C.c_char_p, C.c_int]
     if lib.tb_abi_version() != 1:
         raise RuntimeError("libtritonblas_amd.so ABI version mismatch")
     _lib = lib
     return lib
+
+
+def debug_option(name: str, value: int):
+    """Set one of the library's tuning / test hooks (see ``tb_debug_option`` in the header)."""
+    check(load().tb_debug_option(name.encode(), int(value)), "tb_debug_option")
+
+
+def workspace_layout():
+    """(counters_offset, flags_offset) of a workspace, in bytes."""
+    a, b = C.c_size_t(), C.c_size_t()
+    check(load().tb_workspace_layout(C.byref(a), C.byref(b)), "tb_workspace_layout")
+    return int(a.value), int(b.value)
 
 
 def status_string(status: int) -> str:

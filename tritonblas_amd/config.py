@@ -1,11 +1,17 @@
 """Launch state kept between calls: one device workspace that holds the work-stealing queue
 counters or the Stream-K flags + partial tiles (reference include/tritonblas/config.py:10-134).
 
-Layout of the workspace (bytes): [0, 256) control words (status, done counter); then either
-``num_xcd * counters_per_xcd`` queue counters, one per 256-byte line (work stealing), or ``grid``
-32-bit flags followed by ``grid`` fp32 partial tiles (Stream-K).  Stream-K flags carry the launch
-epoch, so nothing has to be cleared between launches; the work-stealing queues are rearmed by the
-kernel itself.  ``reset()`` is still available after an aborted launch.
+Layout of the workspace (bytes, ``tb_workspace_layout``): [0, 256) control words (status, done
+counter); the work-stealing queue counters, one per 256-byte line; the Stream-K flags (one 32-bit word
+per workgroup) followed by the fp32 partial tiles.  The regions are disjoint, so Stream-K and
+work-stealing launches may share one config in any order.  Stream-K flags carry the launch epoch, so
+nothing has to be cleared between launches; the work-stealing queues are rearmed by the kernel itself.
+``reset()`` is still available after an aborted launch.
+
+A Stream-K owner that waits for a partner's partial tile longer than ``spin_limit`` polls (the partner
+is not resident: another kernel holds its CU, or the stream is CU-masked) gives up: it stores its tile as
+NaN and sets the status word.  The launch itself cannot report this -- it is asynchronous -- so a caller
+that shares the device calls ``check()`` (which synchronises) when it wants to know.
 """
 import torch
 
@@ -34,6 +40,7 @@ class MatmulConfig:
         self.global_atomic = global_atomic
         self.hierarchical = hierarchical
         self.epoch = 0
+        self.spin_limit = 0     # Stream-K: polls per wait before an owner gives up (0: the library's 2**24)
 
     @property
     def mask(self):
@@ -56,30 +63,70 @@ class MatmulConfig:
         return self.workspace
 
     def next_epoch(self) -> int:
-        self.epoch = (self.epoch % 0x7FFFFFFF) + 1
+        """Epochs only count upwards; before they would wrap the workspace is cleared."""
+        if self.epoch >= 0x7FFFFFFF:
+            self.workspace.zero_()
+            self.epoch = 0
+        self.epoch += 1
         return self.epoch
 
-    # views under the reference's attribute names -------------------------------------------------
+    # views under the reference's attribute names (config.py:32-43) ---------------------------------
+    # The reference keeps one buffer per purpose; here they are windows into the one workspace.  The
+    # kernels do not use a global counter, per-iteration counters or "done" bytes: those names return
+    # empty tensors so that code which only resets them keeps working.
+    def _region(self, lo, hi, dtype=torch.int32):
+        ws = self.workspace
+        if ws is None or ws.numel() < hi:
+            return torch.empty(0, dtype=dtype, device=self.device)
+        return ws[lo:hi].view(dtype)
+
     @property
     def tile_counter(self):
-        return self.workspace[_CTL_BYTES:].view(torch.int32)
+        counters, flags = _lib.workspace_layout()
+        return self._region(counters, flags)
+
+    streamk_tile_counter = tile_counter
 
     @property
     def locks(self):
+        _, flags = _lib.workspace_layout()
         grid = self.selector.sk_grid if self.selector is not None else 0
-        return self.workspace[_CTL_BYTES:_CTL_BYTES + 4 * grid].view(torch.int32)
+        return self._region(flags, flags + 4 * grid)
+
+    sk_locks = locks
 
     @property
     def P(self):
         sel = self.selector
         grid = sel.sk_grid
-        off = _CTL_BYTES + ((grid * 4 + 255) // 256) * 256
+        _, flags = _lib.workspace_layout()
+        off = flags + ((grid * 4 + 255) // 256) * 256
         blk = sel.block_m * sel.block_n
-        return self.workspace[off:off + grid * blk * 4].view(torch.float32).view(grid, blk)
+        return self._region(off, off + grid * blk * 4, torch.float32).view(-1, blk)
+
+    sk_P = P
+
+    @property
+    def global_counter(self):
+        return torch.empty(0, dtype=torch.int32, device=self.device)
+
+    sk_iter_counter = global_counter
+    sk_done = global_counter
 
     def status(self) -> int:
         """Control word 0: non-zero after a Stream-K wait ran into its poll bound (synchronises)."""
         return int(self.workspace[:4].view(torch.int32).item())
+
+    def clear_status(self):
+        self.workspace[:4].zero_()
+
+    def check(self):
+        """Raise if a Stream-K launch on this config gave up waiting for a partial tile (it then wrote
+        NaN tiles).  Synchronises with the device; clears the status."""
+        if self.workspace is not None and self.status() != 0:
+            self.clear_status()
+            raise RuntimeError("tritonblas_amd: a Stream-K launch ran into its poll bound (a partner workgroup was "
+                               "not resident); the tiles it could not finish hold NaN")
 
     def reset(self, streamk: bool = False, work_stealing: bool = False):
         """Clear mutable state (reference config.py:54-75)."""

@@ -27,6 +27,14 @@ enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global mem
 enum : int { CTL_STATUS = 0, CTL_DONE = 1, CTL_WORDS = 64 };
 constexpr int COUNTER_STRIDE = 64;  // ints between queue counters: one 256-byte line each
 
+// Measurement hooks of the K loop (skip the copies or the MFMAs; results are then meaningless) exist
+// only in builds with -DTB_LAB_HOOKS; a shipped kernel cannot be told to skip work.
+#ifdef TB_LAB_HOOKS
+#define TB_LAB(p, bit) (((p).debug & (bit)) != 0)
+#else
+#define TB_LAB(p, bit) false
+#endif
+
 struct GemmParams {
   const uint8_t* A;
   const uint8_t* B;
@@ -54,7 +62,7 @@ struct GemmParams {
   int32_t group_m, num_xcds, chunk;
   int32_t panel_n;               // tile order: column panels of this many tiles, swept top to bottom (0: one panel)
   int32_t mode;
-  int32_t debug;                 // tuning experiments: bit0 skip global->LDS copies, bit1 skip MFMA work
+  int32_t debug;                 // measurement builds only (TB_LAB_HOOKS): bit0 skip global->LDS copies, bit1 skip MFMA work
   // Stream-K
   int32_t sk_tiles;
   float* P;
@@ -742,13 +750,13 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
             if (grp >= g0 + 2 && grp * T::SCG < it1) sc_dma(grp);   // (older than the operand copies below)
           }
         }
-        if (it + S < it1 && !(p.debug & 1)) {
+        if (it + S < it1 && !TB_LAB(p, 1)) {
           OA::dma(sa, it + S, lds + stage * T::STAGE_BYTES, li.tid);
           OB::dma(sb, it + S, lds + stage * T::STAGE_BYTES + T::A_BYTES, li.tid);
         }
       };
       auto nothing = []() {};
-      if (p.debug & 2) {
+      if (TB_LAB(p, 2)) {
         boundary();
       } else {
         if constexpr (T::KSUB == 1) {
@@ -785,7 +793,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
         OB::gload(rb, sb, it + 1, p.KU, li.tid);
         load_scales(it + 1, nsca, nscb);
       }
-      if (!(p.debug & 2)) compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
+      if (!TB_LAB(p, 2)) compute(sA0 + cur * T::STAGE_BYTES, sB0 + cur * T::STAGE_BYTES);
       if (has_next) {
         OA::sstore(sA0 + (cur ^ 1) * T::STAGE_BYTES, ra, li.tid);
         OB::sstore(sB0 + (cur ^ 1) * T::STAGE_BYTES, rb, li.tid);
@@ -821,7 +829,19 @@ __device__ __forceinline__ float load_as_f32(const uint8_t* p, int type) {
 
 template <int CT>
 __device__ __forceinline__ void store4(uint8_t* C, int64_t off_el, int64_t sn, v4f v, int nvalid, bool vec) {
-  if constexpr (CT == DT_I8) {
+  if constexpr (CT == DT_FP8) {
+    // fp32 -> e4m3fn: clamp to the largest finite value, then round to nearest even
+    // (the reference's a8w8 oracle, tests/test_matmul_a8w8_lt.py:11-38)
+    float c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c[j] = fminf(fmaxf(v[j], -448.f), 448.f);
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
+    uint8_t* cp = C + off_el;
+    if (vec && nvalid >= 4) { *(uint32_t*)cp = (uint32_t)w; return; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (j < nvalid) cp[j * sn] = (uint8_t)((uint32_t)w >> (8 * j));
+  } else if constexpr (CT == DT_I8) {
     // fp32 -> int8: toward zero, saturated to [-128, 127] (NaN -> 0)
     uint32_t b[4];
 #pragma unroll
@@ -1011,6 +1031,9 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc,
   }
   if constexpr (T::DT == DT_I8) {
     if (p.c_type == DT_I8) { epilogue_t<T, DT_I8>(p, tc, acc, li); return; }
+  }
+  if constexpr (T::DT == DT_FP8) {
+    if (p.c_type == DT_FP8) { epilogue_t<T, DT_FP8>(p, tc, acc, li); return; }
   }
   if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);
   else if (p.c_type == DT_F16) epilogue_t<T, DT_F16>(p, tc, acc, li);
@@ -1347,12 +1370,22 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
         __syncthreads();
         int ok = s_bcast;
         __syncthreads();
-        if (!ok) { failed = true; break; }
+        if (!ok) {
+          // a partner never published (it is not resident, or the bound is too tight): the tile cannot
+          // be finished.  It is stored as NaN so that nobody mistakes stale memory for a result, and the
+          // status word tells the host.
+          failed = true;
+          const float nanv = __builtin_nanf("");
+#pragma unroll
+          for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < T::TN; ++j) acc[i][j] = v4f{nanv, nanv, nanv, nanv};
+          break;
+        }
         partial_add<T>(p.P + (size_t)nxt * (T::BM * T::BN), acc, li.tid);
         cur_end += sched.q + (nxt < sched.rem ? 1 : 0);
         ++nxt;
       }
-      if (failed) break;
     }
     }
     epilogue<T>(p, w.tc, acc, li, lds);

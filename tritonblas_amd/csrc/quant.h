@@ -21,6 +21,6 @@ struct QuantParams {
   int32_t div_shift;
 };
 
-hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, hipStream_t stream);
+hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, bool force_div64, hipStream_t stream);
 
 }  // namespace tb

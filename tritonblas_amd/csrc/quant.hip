@@ -144,16 +144,15 @@ __global__ __launch_bounds__(256) void quant_kernel(const QuantParams p) {
 }
 
 template <int XT, bool HAD>
-static hipError_t launch_t(const QuantParams& p0, hipStream_t stream) {
+static hipError_t launch_t(const QuantParams& p0, bool force_div64, hipStream_t stream) {
   constexpr int UNROLL = 4;
   QuantParams p = p0;
   const int64_t nc = p.n >> 3;
   const int64_t items = p.m * nc;
   const int64_t per_block = 256 * UNROLL;
   const int64_t grid = (items + per_block - 1) / per_block;
-  // testing hook: TB_QUANT_DIV64=1 takes the kernel for 2^31 items and more at any size
-  const char* env = getenv("TB_QUANT_DIV64");
-  if (items < (1ll << 31) && !(env && atoi(env))) {
+  // (force_div64: testing hook, takes the kernel for 2^31 items and more at any size)
+  if (items < (1ll << 31) && !force_div64) {
     // floor(i / nc) for i < 2^31: with l = ceil(log2 nc) and magic = floor(2^(31+l) / nc) + 1 < 2^32,
     // (i * magic) >> (31 + l) is exact; the kernel takes the high product word and shifts by l - 1
     int l = 0;
@@ -167,10 +166,10 @@ static hipError_t launch_t(const QuantParams& p0, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, hipStream_t stream) {
-  if (x_type == QT_BF16) return hadamard ? launch_t<QT_BF16, true>(p, stream) : launch_t<QT_BF16, false>(p, stream);
-  if (x_type == QT_F16) return hadamard ? launch_t<QT_F16, true>(p, stream) : launch_t<QT_F16, false>(p, stream);
-  return hadamard ? launch_t<QT_F32, true>(p, stream) : launch_t<QT_F32, false>(p, stream);
+hipError_t launch_quant(const QuantParams& p, int x_type, bool hadamard, bool force_div64, hipStream_t stream) {
+  if (x_type == QT_BF16) return hadamard ? launch_t<QT_BF16, true>(p, force_div64, stream) : launch_t<QT_BF16, false>(p, force_div64, stream);
+  if (x_type == QT_F16) return hadamard ? launch_t<QT_F16, true>(p, force_div64, stream) : launch_t<QT_F16, false>(p, force_div64, stream);
+  return hadamard ? launch_t<QT_F32, true>(p, force_div64, stream) : launch_t<QT_F32, false>(p, force_div64, stream);
 }
 
 }  // namespace tb

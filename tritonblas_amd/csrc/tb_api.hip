@@ -65,6 +65,47 @@ int current_hw(tb_hw* out) {
   return TB_OK;
 }
 
+// Tuning and test hooks.  The TB_* environment variables are read once, when the library first needs
+// them; tb_debug_option() changes a hook afterwards (tests switch kernels that way).  Nothing on the
+// launch path calls getenv.
+struct Hooks {
+  int waves = 0;                // TB_WAVES=<wm><wn>[<stages>]: picks among variants that share a tile shape
+  int no_mxlds = 0;             // TB_NO_MXLDS=1: fp4 scales straight from global memory (gather kernel)
+  int no_cline = 0;             // TB_NO_CLINE=1: element-wise C stores
+  int no_skinny = 0, skinny = 0;  // TB_NO_SKINNY / TB_SKINNY: force the small-M kernel choice
+  int grid = 0;                 // TB_GRID=<n>: workgroups of a persistent / grouped launch
+  int panel = -1;               // TB_PANEL=<n>: column panel width of the tile order (-1: the library's)
+  int no_column_split = 0, force_column_split = 0;
+  int quant_div64 = 0;          // TB_QUANT_DIV64=1: the quantiser's kernel for 2^31 items and more at any size
+  int lab = 0;                  // TB_DEBUG=<bits>: only acted on by kernels built with TB_LAB_HOOKS
+};
+Hooks g_hooks;
+std::once_flag g_hooks_once;
+std::mutex g_plan_mu;
+uint64_t g_hooks_version = 0;   // bumped whenever a hook changes: cached plans are then stale
+
+int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+void read_hooks() {
+  g_hooks.waves = env_int("TB_WAVES", 0);
+  g_hooks.no_mxlds = env_int("TB_NO_MXLDS", 0);
+  g_hooks.no_cline = env_int("TB_NO_CLINE", 0);
+  g_hooks.no_skinny = env_int("TB_NO_SKINNY", 0);
+  g_hooks.skinny = env_int("TB_SKINNY", 0);
+  g_hooks.grid = env_int("TB_GRID", 0);
+  g_hooks.panel = env_int("TB_PANEL", -1);
+  g_hooks.no_column_split = env_int("TB_NO_COLUMN_SPLIT", 0);
+  g_hooks.force_column_split = env_int("TB_FORCE_COLUMN_SPLIT", 0);
+  g_hooks.quant_div64 = env_int("TB_QUANT_DIV64", 0);
+  g_hooks.lab = env_int("TB_DEBUG", 0);
+}
+const Hooks& hooks() {
+  std::call_once(g_hooks_once, read_hooks);
+  return g_hooks;
+}
+
 void variant_table(int dt, const Variant** v, int* n) {
   switch (dt) {
     case TB_F16: *v = g_variants_f16; *n = g_num_variants_f16; break;
@@ -101,9 +142,7 @@ const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, 
   variant_table(dt, &v, &n);
   // the hand-scheduled 4-wave kernels run K steps in pairs and have no Stream-K form
   auto usable = [&](const Variant& x) { return !x.k_step_pairs || (!need_sk && k > 0 && k % (2 * (int64_t)x.bk) == 0); };
-  // tuning hook: TB_WAVES=<wm><wn>[<stages>] picks among variants that share a tile shape
-  const char* wenv = getenv("TB_WAVES");
-  const int want = wenv ? atoi(wenv) : 0;
+  const int want = hooks().waves;
   if (want && fast)
     for (int i = 0; i < n; ++i)
       if (usable(v[i]) && v[i].fast == fast && v[i].alay == alay && v[i].blay == blay && v[i].bm == bm && v[i].bn == bn && v[i].bk == bk &&
@@ -133,7 +172,7 @@ int default_panel_n(int grid, int chunk, int group_m) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : (dt == TB_F32 ? 4 : 1); }
-int c_bytes(int t) { return t == TB_F32 ? 4 : (t == TB_I8 ? 1 : 2); }
+int c_bytes(int t) { return t == TB_F32 ? 4 : ((t == TB_I8 || t == TB_FP8_E4M3) ? 1 : 2); }
 
 // Everything the launch path needs, independent of which public descriptor it came from.
 struct Job {
@@ -158,6 +197,15 @@ struct Job {
   int column_split = 0;
 };
 
+// Workspace layout (bytes): [0, 256) control words | work-stealing queue counters, one 256-byte line
+// each, WS_MAX_LINES lines | Stream-K flags, one word per workgroup | Stream-K partial tiles.  The
+// regions never overlap whatever schedule a launch runs, so one workspace serves Stream-K launches
+// (whose flags are never cleared: they carry epochs) and work-stealing launches (whose counters must
+// be zero when a launch starts) in any order.
+constexpr size_t WS_MAX_LINES = 520;   // 8 XCDs x 64 slots, a shared pool, spare
+constexpr size_t WS_COUNTERS_OFF = CTL_WORDS * 4;
+constexpr size_t WS_FLAGS_OFF = WS_COUNTERS_OFF + WS_MAX_LINES * COUNTER_STRIDE * 4;
+
 struct Plan {
   const Variant* v = nullptr;
   GemmParams p;
@@ -180,7 +228,9 @@ int kernel_occupancy(const Variant* v, const void* kernel) {
 int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
   if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
-  if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8)) return TB_ERR_BAD_DTYPE;
+  if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8) &&
+      !(j.c_type == TB_FP8_E4M3 && j.dt == TB_FP8_E4M3))
+    return TB_ERR_BAD_DTYPE;
   const int usz = unit_bytes(j.dt);
   const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
   if (j.K % epu) return TB_ERR_BAD_SHAPE;
@@ -218,8 +268,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     // the fast fp4 kernels stage 16 scale bytes per row at a time through LDS with 16-byte copies
     const bool mx_ok = j.mxa_sk == 1 && j.mxb_sk == 1 && (j.K / 32) % 16 == 0 && j.mxa_sr % 16 == 0 && j.mxb_sr % 16 == 0 &&
                        ((uintptr_t)j.mxa % 16) == 0 && ((uintptr_t)j.mxb % 16) == 0;
-    const char* e = getenv("TB_NO_MXLDS");
-    if (!mx_ok || (e && atoi(e))) fast = false;
+    if (!mx_ok || hooks().no_mxlds) fast = false;
   }
   if (fast) {
     // 32-bit offsets inside a tile
@@ -233,7 +282,9 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     int64_t at_once = ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn);
     if (j.schedule == TB_SCHED_STREAMK) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
     if (j.num_groups > 0) at_once = 0;
-    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw, j.schedule == TB_SCHED_STREAMK && j.num_groups == 0, j.K);
+    // (the 4-wave kernels have no Stream-K form and no 8-bit output path)
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw,
+                     (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) || j.c_type == TB_FP8_E4M3, j.K);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
@@ -260,8 +311,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.a_vec = p.b_vec = v->fast;
   const int cb = c_bytes(j.c_type);
   p.c_vec = (j.c_sn == 1 && (j.c_sm % 4 == 0 || j.M == 1) && ((uintptr_t)j.C % (4 * cb)) == 0) ? 1 : 0;
-  p.c_line = (j.c_type != TB_I8 && j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
-  { const char* e = getenv("TB_NO_CLINE"); if (e && atoi(e)) p.c_line = 0; }
+  p.c_line = (j.c_type != TB_I8 && j.c_type != TB_FP8_E4M3 && j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
+  if (hooks().no_cline) p.c_line = 0;
   // (8192x28672x8192 FP8 +0.6 %, 8192^3 bf16 +1.6 %; a small C stays cacheable for whoever reads it next)
   p.c_nt = ((int64_t)j.M * j.N * cb > (int64_t)hw.num_xcd * std::max(hw.l2_bytes, 1 << 20)) ? 1 : 0;
   if (j.dt == TB_FP4_E2M1) {
@@ -279,7 +330,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.group_m = j.group_m > 0 ? j.group_m : std::min(8, (int)p.tiles_m);
   p.num_xcds = j.num_xcds > 0 ? j.num_xcds : hw.num_xcd;
   p.epoch = j.epoch; p.spin_limit = j.spin_limit ? j.spin_limit : (1u << 24);
-  { const char* dbg = getenv("TB_DEBUG"); p.debug = dbg ? atoi(dbg) : 0; }
+  p.debug = hooks().lab;
   p.group_offsets = j.group_offsets; p.num_groups = j.num_groups;
   p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
 
@@ -288,11 +339,9 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     // a handful of rows against a K-major weight: the streaming kernel (no tiles, no workspace) when
     // the model expects it to beat the tile kernel of the requested schedule.  TB_NO_SKINNY=1 / TB_SKINNY=1
     // force the choice (tuning and tests).
-    const char* e = getenv("TB_NO_SKINNY");
-    const char* f = getenv("TB_SKINNY");
     plan->skinny = j.num_groups == 0 && skinny_supported(j.dt, j.M) && alay == LAY_K && blay == LAY_K &&
-                   KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !(e && atoi(e));
-    if (plan->skinny && !(f && atoi(f))) {
+                   KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !hooks().no_skinny && j.c_type != TB_FP8_E4M3;
+    if (plan->skinny && !hooks().skinny) {
       tb_problem pr;
       std::memset(&pr, 0, sizeof(pr));
       pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
@@ -324,12 +373,12 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (bound > INT32_MAX) return TB_ERR_BAD_SHAPE;
     p.total_tiles = (int32_t)bound;
     grid = (int)std::min<int64_t>(bound, resident);
-    { const char* e = getenv("TB_GRID"); if (e && atoi(e) > 0) grid = (int)std::min<int64_t>(bound, atoi(e)); }
+    if (hooks().grid > 0) grid = (int)std::min<int64_t>(bound, hooks().grid);
   } else if (j.schedule == TB_SCHED_PERSISTENT) {
     // a resident grid that loops over the tiles (matmul.py:160-198: for tile_id in range(pid, total, NUM_SMS))
     p.mode = MODE_STATIC;
     grid = (int)std::min<int64_t>(total, j.grid > 0 ? j.grid : resident);
-    { const char* e = getenv("TB_GRID"); if (e && atoi(e) > 0) grid = (int)std::min<int64_t>(total, atoi(e)); }
+    if (hooks().grid > 0) grid = (int)std::min<int64_t>(total, hooks().grid);
   } else if (j.schedule == TB_SCHED_WORK_STEALING) {
     p.mode = MODE_WS;
     grid = j.grid > 0 ? j.grid : (j.cu_mask ? j.cu_mask_len : resident);
@@ -346,8 +395,9 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       return TB_ERR_BAD_SCHEDULE;
     }
     // one counter line per XCD x slot, plus the line of the hierarchical mode's shared pool
-    plan->ws_counters_off = CTL_WORDS * 4;
-    plan->ws_need = plan->ws_counters_off + ((size_t)p.num_xcds * p.counters_per_xcd + 1) * COUNTER_STRIDE * 4;
+    if ((size_t)p.num_xcds * p.counters_per_xcd + 1 > WS_MAX_LINES) return TB_ERR_BAD_SCHEDULE;
+    plan->ws_counters_off = WS_COUNTERS_OFF;
+    plan->ws_need = WS_FLAGS_OFF;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
     // (a requested grid that cannot be co-resident for the kernel that really runs -- the caller sized it
@@ -375,7 +425,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       // nothing to share: the same tiles on the whole-tile kernel (identical results, no workspace)
       p.mode = MODE_STATIC;
     } else {
-      plan->ws_flags_off = CTL_WORDS * 4;
+      plan->ws_flags_off = WS_FLAGS_OFF;
       plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
       plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
     }
@@ -385,7 +435,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (grid <= 0) return TB_ERR_BAD_SHAPE;
   p.chunk = std::min(p.group_m * p.group_m, std::max(1, grid / p.num_xcds));
   p.panel_n = default_panel_n(grid, p.chunk, p.group_m);
-  { const char* e = getenv("TB_PANEL"); if (e) p.panel_n = atoi(e); }
+  if (hooks().panel >= 0) p.panel_n = hooks().panel;
   plan->grid = grid;
   plan->v = v;
   return TB_OK;
@@ -393,12 +443,84 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
 
 int run_plan(const Job& j, Plan& plan, hipStream_t stream);
 
+// ---- plan cache ------------------------------------------------------------------------------------
+// A plan (kernel variant, grid, tile order, schedule parameters) depends on the sizes, strides, types
+// and options of a job and on the alignment of its pointers, not on the pointers themselves.  The
+// launch path keeps the last plans it made and only refreshes the pointers, so a repeated call does not
+// score tiles again (a persistent tb_gemm that considers a column split makes three plans and prices
+// two sub-problems).
+struct PlanKey {
+  int64_t v[30];
+  bool operator==(const PlanKey& o) const { return std::memcmp(v, o.v, sizeof(v)) == 0; }
+};
+PlanKey plan_key(const Job& j, int dev) {
+  PlanKey k;
+  std::memset(&k, 0, sizeof(k));
+  auto al = [](const void* q) { return (int64_t)((uintptr_t)q & 255) | (q ? 256 : 0); };
+  int i = 0;
+  k.v[i++] = ((int64_t)j.dt) | ((int64_t)j.c_type << 8) | ((int64_t)j.bias_type << 16) | ((int64_t)j.schedule << 24) | ((int64_t)dev << 32);
+  k.v[i++] = j.M; k.v[i++] = j.N; k.v[i++] = j.K;
+  k.v[i++] = j.a_sr; k.v[i++] = j.a_sk; k.v[i++] = j.b_sr; k.v[i++] = j.b_sk; k.v[i++] = j.c_sm; k.v[i++] = j.c_sn;
+  k.v[i++] = j.mxa_sr; k.v[i++] = j.mxa_sk; k.v[i++] = j.mxb_sr; k.v[i++] = j.mxb_sk; k.v[i++] = j.bias_stride;
+  k.v[i++] = ((int64_t)j.bm) | ((int64_t)j.bn << 16) | ((int64_t)j.bk << 32) | ((int64_t)j.group_m << 48);
+  k.v[i++] = ((int64_t)j.num_xcds) | ((int64_t)j.grid << 16) | ((int64_t)j.counters_per_xcd << 48);
+  k.v[i++] = ((int64_t)j.ws_mode) | ((int64_t)j.ws_local << 8) | ((int64_t)j.cu_mask_len << 40);
+  k.v[i++] = j.ws_global;
+  k.v[i++] = ((int64_t)j.num_groups) | ((int64_t)j.grp_phase << 16) | ((int64_t)j.grp_big << 24) | ((int64_t)j.grp_thr << 40) | ((int64_t)j.grp_auto << 56);
+  k.v[i++] = j.b_group_stride; k.v[i++] = j.sb_group_stride;
+  k.v[i++] = al(j.A) | (al(j.B) << 10) | (al(j.C) << 20) | (al(j.mxa) << 30) | (al(j.mxb) << 40) | (al(j.bias) << 50);
+  k.v[i++] = (j.sa ? 1 : 0) | (j.sb ? 2 : 0) | (j.cu_mask ? 4 : 0) | (j.group_offsets ? 8 : 0) | ((int64_t)(j.column_split & 3) << 4);
+  k.v[i++] = (int64_t)g_hooks_version;
+  return k;
+}
+// the fields of a plan that name memory or change from call to call
+void refresh_plan(const Job& j, Plan* plan) {
+  GemmParams& p = plan->p;
+  p.A = (const uint8_t*)j.A; p.B = (const uint8_t*)j.B; p.C = (uint8_t*)j.C;
+  p.sa = j.sa; p.sb = j.sb; p.bias = (const uint8_t*)j.bias;
+  p.mxa = (const uint8_t*)j.mxa; p.mxb = (const uint8_t*)j.mxb;
+  p.group_offsets = j.group_offsets;
+  p.cu_mask = (p.mode == MODE_WS) ? j.cu_mask : nullptr;
+  p.epoch = j.epoch; p.spin_limit = j.spin_limit ? j.spin_limit : (1u << 24);
+}
+struct CachedPlan { PlanKey key; Plan plan; int status; uint64_t stamp; };
+constexpr int PLAN_CACHE = 32;
+CachedPlan g_plans[PLAN_CACHE];
+int g_plans_used = 0;
+uint64_t g_plan_clock = 0;
+
+int cached_plan(const Job& j, const tb_hw& hw, Plan* out) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lk(g_plan_mu);
+  const PlanKey key = plan_key(j, dev);
+  for (int i = 0; i < g_plans_used; ++i)
+    if (g_plans[i].key == key) {
+      g_plans[i].stamp = ++g_plan_clock;
+      if (g_plans[i].status != TB_OK) return g_plans[i].status;
+      *out = g_plans[i].plan;
+      refresh_plan(j, out);
+      return TB_OK;
+    }
+  Plan plan;
+  const int st = make_plan(j, hw, true, &plan);
+  int slot = g_plans_used;
+  if (g_plans_used < PLAN_CACHE) ++g_plans_used;
+  else {
+    slot = 0;
+    for (int i = 1; i < PLAN_CACHE; ++i) if (g_plans[i].stamp < g_plans[slot].stamp) slot = i;
+  }
+  g_plans[slot].key = key; g_plans[slot].plan = plan; g_plans[slot].status = st; g_plans[slot].stamp = ++g_plan_clock;
+  if (st == TB_OK) *out = plan;
+  return st;
+}
+
 int launch(const Job& j, hipStream_t stream) {
   tb_hw hw;
   int st = current_hw(&hw);
   if (st != TB_OK) return st;
   Plan plan;
-  st = make_plan(j, hw, true, &plan);
+  st = cached_plan(j, hw, &plan);
   if (st != TB_OK) return st;
   return run_plan(j, plan, stream);
 }
@@ -411,6 +533,9 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
   }
   if (plan.ws_need) {
     if (!j.workspace || j.workspace_bytes < plan.ws_need || ((uintptr_t)j.workspace & 255)) return TB_ERR_WORKSPACE;
+    // Stream-K flags carry the launch epoch and are never cleared: epoch 0 is what a fresh, zeroed
+    // workspace holds in every flag, so a launch tagged 0 would take unpublished partial tiles for published
+    if (p.mode == MODE_SK && j.epoch == 0) return TB_ERR_BAD_ARGUMENT;
     uint8_t* ws = (uint8_t*)j.workspace;
     p.ctl = (uint32_t*)ws;
     if (p.mode == MODE_WS) p.counters = (int32_t*)(ws + plan.ws_counters_off);
@@ -428,21 +553,17 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
 // whole rounds run with the planned tile and the remaining columns as a problem of their own, with the
 // tile the model picks for them (usually a smaller one that spreads over all CUs).  Both launches write
 // disjoint column ranges of C on the same stream.
-int launch_columns(const Job& j, hipStream_t stream) {
-  const char* off = getenv("TB_NO_COLUMN_SPLIT");
-  if (j.schedule != TB_SCHED_PERSISTENT || j.column_split != 0 || j.grid > 0 || j.num_groups > 0 || (off && atoi(off)))
-    return launch(j, stream);
-  tb_hw hw;
-  int st = current_hw(&hw);
-  if (st != TB_OK) return st;
-  Plan whole;
-  st = make_plan(j, hw, true, &whole);
-  if (st != TB_OK) return st;
+struct SplitChoice { PlanKey key; int64_t n1; uint64_t stamp; };   // n1 = 0: one launch
+SplitChoice g_splits[PLAN_CACHE];
+int g_splits_used = 0;
+
+// columns [0, n1) keep the planned tile, the rest becomes a problem of its own; 0 = do not split
+int64_t column_split_point(const Job& j, const tb_hw& hw, const Plan& whole) {
   const Variant* v = whole.v;
   const int64_t total = whole.p.total_tiles, G = whole.grid, tiles_m = whole.p.tiles_m, tiles_n = whole.p.tiles_n;
-  if (whole.skinny || whole.p.mode != MODE_STATIC || !v->fast || total <= G || total % G == 0) return run_plan(j, whole, stream);
+  if (whole.skinny || whole.p.mode != MODE_STATIC || !v->fast || total <= G || total % G == 0) return 0;
   const int64_t tn1 = (total / G) * G / tiles_m;
-  if (tn1 <= 0 || tn1 >= tiles_n) return run_plan(j, whole, stream);
+  if (tn1 <= 0 || tn1 >= tiles_n) return 0;
   const int64_t n1 = tn1 * v->bn, n2 = j.N - n1;
   tb_problem pr;
   std::memset(&pr, 0, sizeof(pr));
@@ -455,22 +576,54 @@ int launch_columns(const Job& j, hipStream_t stream) {
   pr.n = n2;
   tb_selection rest;
   auto infos = tile_infos(j.dt);
-  if (select_tile(pr, hw, infos.data(), (int)infos.size(), &rest) != TB_OK) return run_plan(j, whole, stream);
+  if (select_tile(pr, hw, infos.data(), (int)infos.size(), &rest) != TB_OK) return 0;
   // (testing hook: TB_FORCE_COLUMN_SPLIT=1 splits whatever the model says)
-  const char* force = getenv("TB_FORCE_COLUMN_SPLIT");
-  if (!(force && atoi(force)) && t_first + rest.est_total_us > 0.97 * t_whole) return run_plan(j, whole, stream);
+  if (!hooks().force_column_split && t_first + rest.est_total_us > 0.97 * t_whole) return 0;
+  return n1;
+}
+
+int launch_columns(const Job& j, hipStream_t stream) {
+  if (j.schedule != TB_SCHED_PERSISTENT || j.column_split != 0 || j.grid > 0 || j.num_groups > 0 || hooks().no_column_split)
+    return launch(j, stream);
+  tb_hw hw;
+  int st = current_hw(&hw);
+  if (st != TB_OK) return st;
+  Plan whole;
+  st = cached_plan(j, hw, &whole);
+  if (st != TB_OK) return st;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  int64_t n1 = -1;
+  {
+    std::lock_guard<std::mutex> lk(g_plan_mu);
+    const PlanKey key = plan_key(j, dev);
+    for (int i = 0; i < g_splits_used && n1 < 0; ++i)
+      if (g_splits[i].key == key) { n1 = g_splits[i].n1; g_splits[i].stamp = ++g_plan_clock; }
+    if (n1 < 0) {
+      n1 = column_split_point(j, hw, whole);
+      int slot = g_splits_used;
+      if (g_splits_used < PLAN_CACHE) ++g_splits_used;
+      else {
+        slot = 0;
+        for (int i = 1; i < PLAN_CACHE; ++i) if (g_splits[i].stamp < g_splits[slot].stamp) slot = i;
+      }
+      g_splits[slot].key = key; g_splits[slot].n1 = n1; g_splits[slot].stamp = ++g_plan_clock;
+    }
+  }
+  if (n1 <= 0) return run_plan(j, whole, stream);
+  const Variant* v = whole.v;
   const int usz = unit_bytes(j.dt);
   Job a = j, b = j;
   a.N = n1; a.bm = v->bm; a.bn = v->bn; a.bk = v->bk;
-  b.N = n2; b.bm = b.bn = b.bk = 0; b.group_m = 0;
+  b.N = j.N - n1; b.bm = b.bn = b.bk = 0; b.group_m = 0;
   b.B = (const uint8_t*)j.B + n1 * j.b_sr * usz;
   b.C = (uint8_t*)j.C + n1 * j.c_sn * c_bytes(j.c_type);
   if (j.sb) b.sb = j.sb + n1;
   if (j.bias) b.bias = (const uint8_t*)j.bias + n1 * j.bias_stride * (j.bias_type == TB_F32 ? 4 : 2);
   if (j.mxb) b.mxb = (const uint8_t*)j.mxb + n1 * j.mxb_sr;
   Plan pa, pb;
-  st = make_plan(a, hw, true, &pa);
-  if (st == TB_OK) st = make_plan(b, hw, true, &pb);
+  st = cached_plan(a, hw, &pa);
+  if (st == TB_OK) st = cached_plan(b, hw, &pb);
   if (st != TB_OK || pa.v != v) return run_plan(j, whole, stream);   // (the split must not change what the main part runs)
   st = run_plan(a, pa, stream);
   if (st != TB_OK) return st;
@@ -542,6 +695,25 @@ int tb_hierarchical_split(int64_t total_tiles, int32_t hw_cus, int32_t num_xcds,
 int tb_default_panel(int32_t grid, int32_t chunk, int32_t group_m) {
   if (grid <= 0 || chunk <= 0 || group_m <= 0) return TB_ERR_BAD_ARGUMENT;
   return default_panel_n(grid, chunk, group_m);
+}
+
+int tb_debug_option(const char* name, int value) {
+  if (!name) return TB_ERR_NULL_POINTER;
+  (void)hooks();
+  std::lock_guard<std::mutex> lk(g_plan_mu);
+  struct { const char* n; int* p; } table[] = {
+      {"waves", &g_hooks.waves}, {"no_mxlds", &g_hooks.no_mxlds}, {"no_cline", &g_hooks.no_cline},
+      {"no_skinny", &g_hooks.no_skinny}, {"skinny", &g_hooks.skinny}, {"grid", &g_hooks.grid}, {"panel", &g_hooks.panel},
+      {"no_column_split", &g_hooks.no_column_split}, {"force_column_split", &g_hooks.force_column_split}, {"quant_div64", &g_hooks.quant_div64}, {"lab", &g_hooks.lab}};
+  for (auto& t : table)
+    if (std::strcmp(t.n, name) == 0) { *t.p = value; ++g_hooks_version; return TB_OK; }
+  return TB_ERR_BAD_ARGUMENT;
+}
+
+int tb_workspace_layout(size_t* counters_offset, size_t* flags_offset) {
+  if (!counters_offset || !flags_offset) return TB_ERR_NULL_POINTER;
+  *counters_offset = WS_COUNTERS_OFF; *flags_offset = WS_FLAGS_OFF;
+  return TB_OK;
 }
 
 const char* tb_status_string(int status) {
@@ -666,13 +838,13 @@ int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
   int st = current_hw(&hw);
   if (st != TB_OK) return st;
   Plan first, second;
-  st = make_plan(j, hw, true, &first);
+  st = cached_plan(j, hw, &first);
   if (st != TB_OK) return st;
   if (first.p.grp_phase != 1) return run_plan(j, first, (hipStream_t)stream);
   Job j2 = j;
   j2.bm = kGroupedSmallBM; j2.bn = kGroupedSmallBN; j2.bk = kGroupedSmallBK;
   j2.grp_phase = 2; j2.grp_big = first.p.grp_big;
-  st = make_plan(j2, hw, true, &second);
+  st = cached_plan(j2, hw, &second);
   if (st != TB_OK) return st;
   first.p.grp_small_bm = second.p.grp_small_bm = second.v->bm;
   first.p.grp_other_tn = second.p.tiles_n; first.p.grp_other_grid = second.grid;
@@ -693,7 +865,7 @@ int tb_hadamard_mxfp4_quant(const tb_quant_desc* d, void* stream) {
   QuantParams p;
   p.x = (const uint8_t*)d->x; p.codes = (uint8_t*)d->codes; p.scales = (uint8_t*)d->scales;
   p.m = d->m; p.n = d->n; p.x_stride = d->x_stride_m; p.codes_stride = d->codes_stride_m; p.scales_stride = d->scales_stride_m;
-  hipError_t e = launch_quant(p, d->x_type, d->hadamard != 0, (hipStream_t)stream);
+  hipError_t e = launch_quant(p, d->x_type, d->hadamard != 0, hooks().quant_div64 != 0, (hipStream_t)stream);
   if (e != hipSuccess) return TB_ERR_LAUNCH;
   return TB_OK;
 }

@@ -16,6 +16,21 @@ from .origami import OrigamiMatmulSelector
 
 _SELECTOR_CACHE = {}
 _SELECTOR_CACHE_MAX = 4096
+# Launch state for entry points that are called without a MatmulConfig (tb.matmul(..., enable_streamk=True)
+# and friends): one workspace per (device, stream), grown on demand.  Epoch tags make zeroing between
+# launches unnecessary, and launches on one stream are ordered, so they can share it.
+_STREAM_CONFIGS = {}
+
+
+def _stream_config(dev) -> MatmulConfig:
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    cfg = _STREAM_CONFIGS.get(key)
+    if cfg is None:
+        if len(_STREAM_CONFIGS) >= 64:
+            _STREAM_CONFIGS.clear()
+        cfg = MatmulConfig(device=dev, workspace=None)
+        _STREAM_CONFIGS[key] = cfg
+    return cfg
 
 
 def _make_matmul_selector(M, N, K, a_dtype, b_dtype, c_dtype, device, mx_block_size=0, streamk=False,
@@ -129,10 +144,11 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
         need = lib.tb_workspace_bytes(d)
         if need > 0:
             if config is None:
-                config = MatmulConfig(device=dev, workspace=None, selector=selector)
+                config = _stream_config(dev)
             ws = config.ensure(need)
             d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
             d.epoch = config.next_epoch()
+            d.spin_limit = int(getattr(config, "spin_limit", 0) or 0)
     with _on_device(dev):
         _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
     return c
