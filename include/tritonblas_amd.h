@@ -169,6 +169,17 @@ int tb_gemm(const tb_gemm_desc* desc, void* stream);
 /* Bytes of workspace tb_gemm needs for this descriptor (0 for the persistent schedule). */
 size_t tb_workspace_bytes(const tb_gemm_desc* desc);
 
+/* tb_gemm without a workspace from the caller and without any allocation: the queue counters, Stream-K
+ * flags and partial tiles live in a buffer of TB_STATIC_WORKSPACE_BYTES that is part of the library's
+ * device image (every GPU the library runs on holds it until the process ends).  desc->workspace,
+ * workspace_bytes and epoch are ignored (the library keeps its own epoch per device); a launch that
+ * needs more than TB_STATIC_WORKSPACE_BYTES is refused with TB_ERR_WORKSPACE.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory where they launch -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid it.  All calls on one GPU share the buffer:
+ * calls that may overlap in time (different streams) race; calls on one stream do not. */
+#define TB_STATIC_WORKSPACE_BYTES (16u << 20)
+int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream);
+
 /* Byte offsets of the regions of a workspace: [0, 256) control words -- word 0 is the status (set to 1
  * when a Stream-K wait ran into spin_limit: the tile concerned was then stored as NaN; cleared only by the
  * caller), word 1 counts finished work-stealing workgroups; *counters_offset: work-stealing queue

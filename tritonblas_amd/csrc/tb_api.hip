@@ -630,6 +630,35 @@ int launch_columns(const Job& j, hipStream_t stream) {
   return run_plan(b, pb, stream);
 }
 
+// ---- the library's own scratch buffer ---------------------------------------------------------------
+// tb_gemm_static_workspace() runs the schedules that need a workspace without one from the caller: the
+// queue counters, Stream-K flags and partial tiles live in this array.  Each device holds its own copy
+// at its own address; the array's name is only a handle for hipGetSymbolAddress in host code.
+constexpr size_t SCRATCH_BYTES = TB_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+struct ScratchState {
+  void* ptr = nullptr;
+  int status = TB_ERR_NO_DEVICE;
+  uint32_t epoch = 0;
+};
+ScratchState g_scratch[MAX_DEVICES];
+std::once_flag g_scratch_once[MAX_DEVICES];
+std::mutex g_scratch_mu;
+
+void init_scratch(int dev) {
+  void* ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // (the current device's copy)
+  if (e != hipSuccess || !ptr) { (void)hipGetLastError(); g_scratch[dev].status = TB_ERR_NO_DEVICE; return; }
+  g_scratch[dev].ptr = ptr;
+  g_scratch[dev].status = TB_OK;
+}
+
+// clears words [0, n) of a buffer (used instead of a memset node, which a caller's graph capture must not record)
+__global__ void fill_zero_kernel(uint32_t* ptr, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) ptr[i] = 0u;
+}
+
 int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
@@ -772,6 +801,33 @@ int tb_gemm(const tb_gemm_desc* desc, void* stream) {
   if (st != TB_OK) return st;
   if (!j.A || !j.B || !j.C) return TB_ERR_NULL_POINTER;
   if (desc->column_split < -1 || desc->column_split > 0) return TB_ERR_BAD_ARGUMENT;
+  return launch_columns(j, (hipStream_t)stream);
+}
+
+int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream) {
+  Job j;
+  int st = job_from_gemm(desc, &j);
+  if (st != TB_OK) return st;
+  if (!j.A || !j.B || !j.C) return TB_ERR_NULL_POINTER;
+  if (desc->column_split < -1 || desc->column_split > 0) return TB_ERR_BAD_ARGUMENT;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return TB_ERR_NO_DEVICE;
+  std::call_once(g_scratch_once[dev], init_scratch, dev);
+  ScratchState& sc = g_scratch[dev];
+  if (sc.status != TB_OK) return sc.status;
+  j.workspace = sc.ptr;
+  j.workspace_bytes = SCRATCH_BYTES;   // (a launch that needs more is refused with TB_ERR_WORKSPACE)
+  {
+    // the array keeps the last call's contents: Stream-K flags are told apart by a per-device epoch that
+    // only counts upwards; when it would wrap, the flags are cleared first (the queue counters rearm themselves)
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (sc.epoch == 0xFFFFFFFFu) {
+      hipLaunchKernelGGL(fill_zero_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, (uint32_t*)sc.ptr, SCRATCH_BYTES / 4);
+      if (hipGetLastError() != hipSuccess) return TB_ERR_LAUNCH;
+      sc.epoch = 0;
+    }
+    j.epoch = ++sc.epoch;
+  }
   return launch_columns(j, (hipStream_t)stream);
 }
 
