@@ -126,6 +126,34 @@ def test_fp4_four_wave_kernel(m, n, k, tb_option):
     assert torch.equal(outs[22].view(torch.int16), outs[24].view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (512, 768, 512), (300, 500, 384), (1, 300, 256), (2048, 1280, 1024)])
+def test_16bit_four_wave_kernel(dtype, m, n, k, tb_option):
+    """bf16 / fp16 with K-major operands (the TN layout): oracle parity, bit-equality with the 8-wave
+    kernel, and a per-column bias through the general epilogue."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import persistent_matmul_lt
+    _say(f"w4 {dtype} {m}x{n}x{k}")
+    g = torch.Generator().manual_seed(76)
+    a_cpu = (torch.randn(m, k, generator=g) * 0.5).to(dtype)
+    bt_cpu = (torch.randn(n, k, generator=g) * 0.5).to(dtype)
+    bias = torch.randn(n, generator=g).to(dtype)
+    a, b = a_cpu.cuda(), bt_cpu.cuda().T
+    want = OG.ref_gemm(a_cpu, bt_cpu.T, torch.float32)
+    for with_bias in (False, True):
+        outs = {}
+        for waves in (22, 24):
+            tb_option("waves", waves)
+            sel = tb.OrigamiMatmulSelector(m, n, k, dtype, dtype, dtype, a.device)
+            sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 64
+            c = torch.full((m, n), float("nan"), dtype=dtype, device="cuda")
+            persistent_matmul_lt(a, b, c, sel, None, bias=bias.cuda() if with_bias else None)
+            outs[waves] = c.cpu()
+        ref = (want + bias.float()[None, :]) if with_bias else want
+        assert OG.rel_fro_error(outs[22].float(), ref.to(dtype).float()) <= 1e-3
+        assert torch.equal(outs[22].view(torch.int16), outs[24].view(torch.int16))
+
+
 # ---- workspace rules --------------------------------------------------------------------------------------
 def test_streamk_then_work_stealing_on_one_config():
     """Stream-K flags and work-stealing counters live in disjoint regions of the workspace: a Stream-K

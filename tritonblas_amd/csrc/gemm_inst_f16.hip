@@ -11,6 +11,8 @@ namespace tb {
   make_variant<Tile<DT_F16, BM, BN, 128, WM, WN, LAY_M, LAY_M, MINB, true, 2>>()
 
 const Variant g_variants_f16[] = {
+    // hand-scheduled 4-wave kernel (K-major operands): taken when K is a multiple of two K steps and no Stream-K tail is asked for
+    make_variant_w4<W4Tile<DT_F16>>(),
     TB_LAYOUTS(256, 256, 2, 4, 1),
     TB_LAYOUTS(128, 128, 2, 2, 2),
     TB_LAYOUTS(64, 64, 2, 2, 4),

@@ -75,13 +75,13 @@ struct W4Lane {
 template <class T>
 __device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, W4TileArgs& t) {
   const int rva = tc.m_lim - tc.m0, rvb = tc.n_lim - tc.n0;
-  const uint32_t sra = (uint32_t)p.a_sr, srb = (uint32_t)p.b_sr;   // bytes (one-byte storage units)
+  const uint32_t sra = (uint32_t)p.a_sr * T::USZ, srb = (uint32_t)p.b_sr * T::USZ;   // row strides in bytes
 #ifdef W4_LAB_SAMETILE
   t.A = p.A;   // measurement build: every tile reads the operands of tile (0, 0) (all copies hit in L2)
   t.B = tc.B;
 #else
-  t.A = p.A + (int64_t)tc.m0 * p.a_sr;
-  t.B = tc.B + (int64_t)tc.n0 * p.b_sr;
+  t.A = p.A + (int64_t)tc.m0 * p.a_sr * T::USZ;
+  t.B = tc.B + (int64_t)tc.n0 * p.b_sr * T::USZ;
 #endif
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -224,7 +224,7 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
-  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4, "element types with a 128-byte K step per MFMA");
+  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16, "element types with a generated K loop");
   __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_ALLOC];
   int& s_bcast = *(int*)(lds + T::LDS_ALLOC - 16);
   const int tid = threadIdx.x;
@@ -294,6 +294,24 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     if constexpr (T::DT == DT_FP8) {
       asm volatile(
 #include "w4_kloop_fp8.inc"
+          : [scbuf] "+s"(scbuf)
+          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
+            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          :
+#include "w4_clobbers.inc"
+      );
+    } else if constexpr (T::DT == DT_BF16) {
+      asm volatile(
+#include "w4_kloop_bf16.inc"
+          : [scbuf] "+s"(scbuf)
+          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
+            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          :
+#include "w4_clobbers.inc"
+      );
+    } else if constexpr (T::DT == DT_F16) {
+      asm volatile(
+#include "w4_kloop_f16.inc"
           : [scbuf] "+s"(scbuf)
           : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
             [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)

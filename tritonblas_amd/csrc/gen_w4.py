@@ -1,13 +1,13 @@
 #!/usr/bin/env python3
 """Writes the hand-scheduled K loop of the 4-wave 256x256 tile kernels (gemm_w4.h) as inline-assembly text.
 
-    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        python3 gen_w4.py fp4 > w4_kloop_fp4.inc
+    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: fp4, bf16, f16)
     python3 gen_w4.py clobbers > w4_clobbers.inc
 
 One workgroup = 4 waves (one per SIMD), wave (wm, wn) owns the 128x128 quarter of a 256x256 output
 tile: 8x8 MFMA tiles of 16x16, i.e. 256 accumulator registers a[0:255]; acc(i, j) of A row block i and
-B row block j sits in a[(8i+j)*4 .. +3].  A K step is 128 bytes of every operand row (128 FP8 values
-or 256 FP4 values); LDS holds two stages of 64 KB: stage s at s*65536, A rows at +0, B rows at +32768,
+B row block j sits in a[(8i+j)*4 .. +3].  A K step is 128 bytes of every operand row (128 FP8 values,
+256 FP4 values or 64 16-bit values); LDS holds two stages of 64 KB: stage s at s*65536, A rows at +0, B rows at +32768,
 row r at r*128 with its eight 16-byte chunks XOR-swizzled (the layout the 8-wave kernels use).  FP4
 adds two 8 KB buffers of E8M0 scales behind the stages (16 scale bytes per row = two K steps).
 
@@ -51,12 +51,16 @@ S_CA, S_CB, S_CSA, S_CSB, S_CNT, S_SCN, S_T, S_SCIN, S_FIRST = 70, 72, 74, 76, 7
 
 
 class Gen:
-    def __init__(self, fp4, dma_every=1, lab=()):
-        self.fp4 = fp4
+    def __init__(self, kind, dma_every=1, lab=()):
+        self.kind = kind                # "fp8" | "fp4" | "bf16" | "f16"
+        self.fp4 = kind == "fp4"        # (the only kind with E8M0 scale operands)
         self.out = []
-        self.nm = 16 if fp4 else 8      # MFMAs per row block
+        self.nm = 8 if kind == "fp8" else 16      # MFMAs per row block (FP8: one of K = 128 per fragment pair; others: two half-K ones)
         self.dma_every = dma_every
         self.lbl = 0
+        # how far (in MFMAs) into row blocks 1 and 5 the two sync points of a K step sit
+        self.xoff = int(os.environ.get("W4GEN_XOFF", str(self.nm // 2)))
+        self.yoff = int(os.environ.get("W4GEN_YOFF", str(self.nm // 2)))
         # measurement builds (W4GEN_LAB=nomfma,nodma,noread,nobar): leave one kind of instruction out to time
         # the rest; results are then meaningless
         self.lab = set(lab)
@@ -142,14 +146,18 @@ class Gen:
 
     def mfma(self, p, i, slot):
         """MFMA number `slot` of row block i: B fragment first (its rows become the output rows a lane holds)"""
-        if not self.fp4:
+        if self.kind == "fp8":
             j = slot
             acc = (i * 8 + j) * 4
             b, a = self.vB(p, j), self.vA(i)
             return f"v_mfma_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 7}], v[{a}:{a + 7}], a[{acc}:{acc + 3}]"
+        # two MFMAs per accumulator and K step, k slice outermost so that the same accumulator comes up
+        # again only eight instructions later
         ks, j = slot // 8, slot % 8
         acc = (i * 8 + j) * 4
         b, a = self.vB(p, j) + 4 * ks, self.vA(i) + 4 * ks
+        if self.kind in ("bf16", "f16"):
+            return f"v_mfma_f32_16x16x32_{self.kind} a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], a[{acc}:{acc + 3}]"
         return (f"v_mfma_scale_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], a[{acc}:{acc + 3}], "
                 f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
 
@@ -196,24 +204,27 @@ class Gen:
         # row block 0
         pre[0] += self.frag_read(self.vA(3), 0, p, 3)
         pre[0].append("s_waitcnt lgkmcnt(6)")
-        # X
+        # X: part of the way into row block 1, so that the read of A fragment 3 (requested when row block 0
+        # started) has had time to return before lgkmcnt(0) asks for it
+        xs = nm + self.xoff
         # (X of step 0: nothing of this tile may be assumed younger than the stores; X of step 1: the
         # steady-state count already demands that the stores are done)
-        pre[nm] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx_other + 4, nx_other + 4 + NST, 0 if p == 0 else nx_other + 4) + ["s_barrier"]
+        pre[xs] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx_other + 4, nx_other + 4 + NST, 0 if p == 0 else nx_other + 4) + ["s_barrier"]
         if p == 1:
-            post[nm].append(f"s_mov_b32 s{S_FIRST}, 0")
-        pre[nm] += self.frag_read(self.vA(4), 0, p, 4)
+            post[xs].append(f"s_mov_b32 s{S_FIRST}, 0")
+        pre[xs] += self.frag_read(self.vA(4), 0, p, 4)
         xops = ops_b + lo + sc
-        span = 4 * nm - 2
+        span = 5 * nm - 2 - xs
         for n, op in enumerate(xops):
-            post[nm + n * span // len(xops)] += op
+            post[xs + n * span // len(xops)] += op
         post[5 * nm - 2] += adv_b
         pre[2 * nm] += self.frag_read(self.vA(5), 0, p, 5)
         pre[3 * nm] += self.frag_read(self.vA(6), 0, p, 6)
         pre[4 * nm] += self.frag_read(self.vA(7), 0, p, 7)
+        # (A fragment 4 was requested at X; fragments 5, 6, 7 are younger)
         pre[4 * nm].append("s_waitcnt lgkmcnt(6)")
         # Y
-        tail0 = BND * nm
+        tail0 = BND * nm + self.yoff
         if p == 0:
             pre[tail0] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx + 4, nx + 4 + NST, nx) + ["s_barrier"]
         else:
@@ -233,8 +244,11 @@ class Gen:
             span = tail // 2
             for n, l in enumerate(lds):
                 post[tail0 + n * span // len(lds)].append(l)
-            post[tail0 + tail // 2] += self.frag_read(self.vA(1), 0, q, 1)
-            post[tail0 + tail * 5 // 6] += self.frag_read(self.vA(2), 0, q, 2)
+            # A fragments 1 and 2 of the next step go where row blocks 5 and 6 read from: behind those
+            a1 = max(tail0 + tail // 2, 6 * nm)
+            a2 = max(tail0 + tail * 5 // 6, 7 * nm)
+            post[a1] += self.frag_read(self.vA(1), 0, q, 1)
+            post[a2] += self.frag_read(self.vA(2), 0, q, 2)
         for n, op in enumerate(hi):
             post[tail0 + n * (tail - 2) // len(hi)] += op
         post[total - 2] += adv_a
@@ -349,7 +363,7 @@ def main():
         return
     import os
     every = int(os.environ.get("W4GEN_DMA_EVERY", "1" if what == "fp8" else "2"))
-    g = Gen(what == "fp4", every, [x for x in os.environ.get("W4GEN_LAB", "").split(",") if x])
+    g = Gen(what, every, [x for x in os.environ.get("W4GEN_LAB", "").split(",") if x])
     g.kloop()
     sys.stdout.write(g.text())
 
