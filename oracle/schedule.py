@@ -133,14 +133,15 @@ def grouped_two_launch_blocks(offsets, phase, big_m, small_rows, block_m):
 
 def grouped_split_pays(offsets, big_m, small_rows, small_m, tiles_n_big, tiles_n_small, grid_big, grid_small):
     """The verdict both launches of a grouped GEMM reach on the device from the row counts: split when
-    2 * rounds(tall tiles of the split plan) + rounds(short tiles) < 2 * rounds(tall tiles of the
+    4 * rounds(tall tiles of the split plan) + 3 * rounds(short tiles) < 4 * rounds(tall tiles of the
     one-launch plan) and there is a short block at all (a round of short tiles streams half a tall
-    round's weight bytes and is priced at half its time).  New work, no reference counterpart."""
+    round's weight bytes but is bound by that stream: measured at three quarters of a tall round).
+    New work, no reference counterpart."""
     one = len(grouped_two_launch_blocks(offsets, 1, big_m, 0, big_m))
     b1 = len(grouped_two_launch_blocks(offsets, 1, big_m, small_rows, big_m))
     b2 = len(grouped_two_launch_blocks(offsets, 2, big_m, small_rows, small_m))
-    cost_one = 2 * cdiv(one * tiles_n_big, grid_big)
-    cost_two = 2 * cdiv(b1 * tiles_n_big, grid_big) + cdiv(b2 * tiles_n_small, grid_small)
+    cost_one = 4 * cdiv(one * tiles_n_big, grid_big)
+    cost_two = 4 * cdiv(b1 * tiles_n_big, grid_big) + 3 * cdiv(b2 * tiles_n_small, grid_small)
     return b2 > 0 and cost_two < cost_one
 
 

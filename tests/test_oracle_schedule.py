@@ -127,13 +127,15 @@ def test_grouped_two_launches_cover_every_row_once(small_rows):
 
 def test_grouped_split_verdicts():
     """Hand-priced cases on 256 compute units, 8 experts of (14336, 4096) weights: 56 column tiles of
-    256, 112 of 128.  Routed counts with five remainders of at most 27 rows: 37 blocks = 9 rounds
-    against 32 blocks = 7 rounds + 560 short tiles = 3 rounds (17 < 18: split).  Remainders of 60
-    rows on four experts: 36 blocks = 8 rounds (16) against 7 rounds + 896 short tiles = 4 rounds (18):
-    one launch.  Equal counts: nothing short, one launch."""
+    256, 112 of 128; a round of tall tiles costs 4, a round of short tiles 3.  Routed counts with five
+    remainders of at most 27 rows: 37 blocks = 9 rounds (36) against 32 blocks = 7 rounds + 560 short
+    tiles = 3 rounds (28 + 9 = 37): one launch.  Remainders of 60 rows on four experts: 36 blocks = 8
+    rounds (32) against 7 rounds + 896 short tiles = 4 rounds (40): one launch.  Equal counts: nothing
+    short, one launch.  One big expert and two single rows: 34 blocks = 8 rounds (32) against 7 rounds +
+    224 short tiles = 1 round (31): split."""
     def verdict(counts):
         return S.grouped_split_pays([0] + list(np.cumsum(counts)), 256, 64, 32, 56, 112, 256, 256)
-    assert verdict([1051, 1035, 1034, 1029, 997, 1019, 991, 1036]) is True
+    assert verdict([1051, 1035, 1034, 1029, 997, 1019, 991, 1036]) is False
     assert verdict([1084, 964] * 4) is False
     assert verdict([1024] * 8) is False
-    assert verdict([8190, 1, 1, 0, 0, 0, 0, 0]) is True      # 34 blocks = 8 rounds (16) against 7 rounds + 1 (15)
+    assert verdict([8190, 1, 1, 0, 0, 0, 0, 0]) is True

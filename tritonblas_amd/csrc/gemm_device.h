@@ -84,7 +84,7 @@ struct GemmParams {
   // partial block of at most grp_thr rows to phase 2, which tiles just those rows with a short tile
   // (a handful of rows would otherwise cost a whole tall tile per column block).  Phase 0: one launch.
   // With grp_auto every workgroup of both launches first prices the two plans from the row counts
-  // (rounds of tall tiles cost 2, rounds of short tiles 1) and both launches act on the same verdict:
+  // (rounds of tall tiles cost 4, rounds of short tiles 3) and both launches act on the same verdict:
   // either the first runs the one-launch table and the second does nothing, or they split the rows.
   int32_t grp_phase, grp_big, grp_thr;
   int32_t grp_auto, grp_small_bm;
@@ -1130,8 +1130,8 @@ __device__ __forceinline__ int grouped_phase(const GemmParams& p, int grid) {
   }
   const int tn_big = p.grp_phase == 1 ? p.tiles_n : p.grp_other_tn, tn_small = p.grp_phase == 1 ? p.grp_other_tn : p.tiles_n;
   const int g_big = p.grp_phase == 1 ? grid : p.grp_other_grid, g_small = p.grp_phase == 1 ? p.grp_other_grid : grid;
-  const int64_t one = 2 * (((int64_t)b0 * tn_big + g_big - 1) / g_big);
-  const int64_t two = 2 * (((int64_t)b1 * tn_big + g_big - 1) / g_big) + ((int64_t)b2 * tn_small + g_small - 1) / g_small;
+  const int64_t one = 4 * (((int64_t)b0 * tn_big + g_big - 1) / g_big);
+  const int64_t two = 4 * (((int64_t)b1 * tn_big + g_big - 1) / g_big) + 3 * (((int64_t)b2 * tn_small + g_small - 1) / g_small);
   const bool split = b2 > 0 && two < one;
   if (p.grp_phase == 1) return split ? 1 : 0;
   return split ? 2 : -1;

@@ -80,7 +80,7 @@ static double family_efficiency(int dt, const TileInfo& v) {
   const int cls = (v.bm < 64 || v.bn < 64) ? 3 : (area >= 256 * 256 ? 0 : (area >= 128 * 128 ? 1 : 2));
   static const double f8[4] = {0.61, 0.46, 0.29, 0.15};     // (128x128: 8192x28672x8192 in 1.72-1.77 ms, 8192^3 in 0.48 ms)
   static const double h16[4] = {0.59, 0.465, 0.22, 0.12};  // (128x128: 8192^3 bf16 in 0.97 ms)
-  static const double f4[4] = {0.45, 0.36, 0.22, 0.10};
+  static const double f4[4] = {0.50, 0.36, 0.22, 0.10};     // (256x256: the 4-wave kernel, 8192x8192x16384 in 0.43-0.47 ms)
   static const double f32[4] = {0.80, 0.75, 0.60, 0.30};   // the fp32 matrix pipe is slow enough to hide everything else
   if (dt == TB_FP8_E4M3 || dt == TB_I8) return f8[cls];
   if (dt == TB_FP4_E2M1) return f4[cls];
