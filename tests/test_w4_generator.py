@@ -1,0 +1,58 @@
+"""The generator of the 4-wave kernels' K loop proves its own wait counts: every `s_waitcnt vmcnt(n)` it
+writes is replayed against the instruction stream of every history a tile can have (first tile of a
+workgroup, after compiled epilogue stores, after a fused epilogue) and must not allow more operations
+in flight than were issued after the copies it waits for."""
+import importlib.util
+import os
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GEN = os.path.join(os.path.dirname(HERE), "tritonblas_amd", "csrc", "gen_w4.py")
+
+
+def _load():
+    spec = importlib.util.spec_from_file_location("gen_w4", GEN)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "f16"])
+def test_wait_counts_hold_for_every_history(kind):
+    gen = _load()
+    slack = gen.Gen(kind).check()
+    assert slack and min(slack.values()) >= 0
+
+
+def test_checker_catches_a_wait_that_is_too_loose():
+    """the same replay with one wait loosened by one must fail"""
+    gen = _load()
+    g = gen.Gen("fp8")
+    parts = g.parts()
+    waits = [o for o in parts["steady1"] if isinstance(o, gen.WaitVm)]
+    assert waits
+    g.parts = lambda: parts
+    for k in waits[0].vals:
+        waits[0].vals[k] += 1
+    with pytest.raises(AssertionError):
+        g.check()
+
+
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16"])
+def test_program_shape(kind):
+    """one MFMA per accumulator tile and K slice in every step; the fused epilogue stores 32 times"""
+    gen = _load()
+    g = gen.Gen(kind)
+    parts = g.parts()
+    per_step = 64 if kind == "fp8" else 128
+    for name in ("first0", "first0_fe", "first1", "steady0", "steady1", "last0", "last1"):
+        assert sum(1 for o in parts[name] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")) == per_step, name
+    stores = [o for o in parts["first0_fe"] if not isinstance(o, gen.WaitVm) and o.text.startswith("global_store")]
+    assert len(stores) == 32
+    assert not any(o.text.startswith("global_store") for o in parts["first0"] if not isinstance(o, gen.WaitVm))
+    # the first K step starts every sum from zero, the others accumulate
+    first = [o.text for o in parts["first0"] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")]
+    assert sum(1 for t in first if t.count("a[") == 1) == 64          # (no accumulator among the sources)
+    steady = [o.text for o in parts["steady0"] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")]
+    assert all(t.count("a[") == 2 for t in steady)

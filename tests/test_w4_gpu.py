@@ -48,7 +48,7 @@ def _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=torch.bfloat16, bias=No
     return c.cpu()
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (256, 256, 2048), (512, 768, 512), (300, 500, 768), (1, 257, 256),
+@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (256, 256, 2048), (512, 768, 512), (300, 500, 768), (1, 257, 512),
                                    (1024, 2048, 1024), (2560, 2304, 512)])
 def test_fp8_four_wave_kernel(m, n, k, tb_option):
     """Whole and ragged tiles, one to many tiles per workgroup (2560x2304 = 90 tiles): oracle parity and
@@ -89,9 +89,11 @@ def test_fp8_four_wave_work_stealing(tb_option):
         assert torch.equal(static.view(torch.int16), ws.view(torch.int16)), f"launch {rep}"
 
 
-def test_fp8_four_wave_needs_an_even_number_of_k_steps(tb_option):
-    """K = 3 steps of 128: the library must fall back to the 8-wave kernel by itself and stay correct."""
-    m, n, k = 512, 512, 384
+@pytest.mark.parametrize("k", [256, 384, 640])
+def test_fp8_four_wave_needs_an_even_number_of_k_steps(k, tb_option):
+    """K = 2, 3 or 5 steps of 128 (the 4-wave kernel runs an even number, at least four): the library must
+    fall back to the 8-wave kernel by itself and stay correct."""
+    m, n = 512, 512
     aq, bq, sa, sb = _fp8_case(m, n, k, 74)
     got = _run_fp8(aq, bq, sa, sb, 0, tb_option)
     want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
@@ -107,7 +109,7 @@ def _fp4_case(m, n, k, seed):
     return torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs), torch.from_numpy(ws)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (256, 256, 4096), (512, 768, 1024), (300, 500, 1536), (2048, 1280, 2048)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 1024), (256, 256, 4096), (512, 768, 1024), (300, 500, 1536), (2048, 1280, 2048)])
 def test_fp4_four_wave_kernel(m, n, k, tb_option):
     import tritonblas_amd as tb
     _say(f"w4 fp4 {m}x{n}x{k}")
@@ -127,7 +129,7 @@ def test_fp4_four_wave_kernel(m, n, k, tb_option):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (512, 768, 512), (300, 500, 384), (1, 300, 256), (2048, 1280, 1024)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (512, 768, 512), (300, 500, 384), (1, 300, 256), (2048, 1280, 1024)])
 def test_16bit_four_wave_kernel(dtype, m, n, k, tb_option):
     """bf16 / fp16 with K-major operands (the TN layout): oracle parity, bit-equality with the 8-wave
     kernel, and a per-column bias through the general epilogue."""
@@ -152,6 +154,85 @@ def test_16bit_four_wave_kernel(dtype, m, n, k, tb_option):
         ref = (want + bias.float()[None, :]) if with_bias else want
         assert OG.rel_fro_error(outs[22].float(), ref.to(dtype).float()) <= 1e-3
         assert torch.equal(outs[22].view(torch.int16), outs[24].view(torch.int16))
+
+
+# ---- epilogue fused into the next tile's K loop -------------------------------------------------------------
+def _launcher(kind, m, n, k, seed):
+    """returns (run, want): run() launches the 256x256 tile kernel the hooks select and returns C on the host"""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import persistent_matmul_lt
+    if kind == "fp8":
+        aq, bq, sa, sb = _fp8_case(m, n, k, seed)
+        a, b, sad, sbd = aq.cuda(), bq.T.contiguous().cuda().T, sa.cuda(), sb.cuda()
+
+        def run():
+            sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.bfloat16, a.device)
+            sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 128
+            c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            persistent_matmul_lt(a, b, c, sel, None, a_scale=sad, b_scale=sbd, quantized=True)
+            return c.cpu()
+        return run, OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
+    if kind == "fp4":
+        xq, wq, xs, ws = _fp4_case(m, n, k, seed)
+        xs[::3, ::2] = 121
+        xd, wd, xsd, wsd = xq.cuda(), wq.cuda(), xs.cuda(), ws.cuda()
+
+        def run():
+            c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            tb.matmul_fp4(xd, wd, c, xsd, wsd, block_m=256, block_n=256, block_k=256)
+            return c.cpu()
+        return run, OG.ref_gemm_fp4(xq, wq, xs, ws, return_fp32=True).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(seed)
+    a_cpu = (torch.randn(m, k, generator=g) * 0.5).bfloat16()
+    bt_cpu = (torch.randn(n, k, generator=g) * 0.5).bfloat16()
+    a, b = a_cpu.cuda(), bt_cpu.cuda().T
+
+    def run():
+        sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.bfloat16, a.device)
+        sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 64
+        c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        persistent_matmul_lt(a, b, c, sel, None)
+        return c.cpu()
+    return run, OG.ref_gemm(a_cpu, bt_cpu.T, torch.float32).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("kind,bk", [("fp8", 128), ("fp4", 256), ("bf16", 64)])
+@pytest.mark.parametrize("m,n,steps,grid", [(512, 768, 4, 1), (512, 768, 6, 2), (300, 500, 8, 1), (1280, 768, 10, 3), (1100, 1300, 4, 2),
+                                            (4096, 8192, 4, 0)])
+def test_fused_epilogue(kind, bk, m, n, steps, grid, tb_option):
+    """A workgroup that runs several tiles stores a full bf16 tile from inside the next tile's first K
+    step.  With 1 to 3 workgroups for 6 to 30 tiles (and 512 tiles on the whole chip), whole and ragged
+    tiles mixed, the result must equal, bit for bit, what the same kernel gives when every tile takes
+    the compiled epilogue (hook lab = 4) and what the 8-wave kernel gives; twice in a row; and it must
+    agree with the oracle."""
+    k = steps * bk
+    _say(f"fused epilogue {kind} {m}x{n}x{k} grid {grid}")
+    run, want = _launcher(kind, m, n, k, 81)
+    tb_option("grid", grid)
+    tb_option("waves", 24)
+    eight = run()
+    tb_option("waves", 22)
+    tb_option("lab", 4)
+    compiled = run()
+    tb_option("lab", 0)
+    fused = run()
+    again = run()
+    assert OG.rel_fro_error(fused.float(), want.float()) <= (1e-3 if kind == "bf16" else TOL_Q)
+    assert torch.equal(compiled.view(torch.int16), eight.view(torch.int16))
+    assert torch.equal(fused.view(torch.int16), compiled.view(torch.int16))
+    assert torch.equal(again.view(torch.int16), fused.view(torch.int16))
+
+
+def test_fused_epilogue_work_stealing(tb_option):
+    """Tiles drawn from the work-stealing queues (which tile follows which is decided at run time) with
+    two workgroups: same bits as the data-parallel launch."""
+    m, n, k = 1280, 1024, 512
+    aq, bq, sa, sb = _fp8_case(m, n, k, 82)
+    tb_option("grid", 2)
+    static = _run_fp8(aq, bq, sa, sb, 22, tb_option)
+    for rep in range(2):
+        ws = _run_fp8(aq, bq, sa, sb, 22, tb_option, work_stealing=True)
+        assert torch.equal(static.view(torch.int16), ws.view(torch.int16)), f"launch {rep}"
 
 
 # ---- workspace rules --------------------------------------------------------------------------------------

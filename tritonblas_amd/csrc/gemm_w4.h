@@ -221,12 +221,19 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
   });
 }
 
+// operands every kind of K loop statement takes
+#define W4_COMMON_OPERANDS                                                                                              \
+  [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [A] "s"(sA), [B] "s"(sB),     \
+      [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst), [fe] "s"(s_fe), \
+      [cprev] "s"(s_cprev), [cstep] "s"(s_cstep)
+
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
   static_assert(T::DT == DT_FP8 || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16, "element types with a generated K loop");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[T::LDS_ALLOC];
-  int& s_bcast = *(int*)(lds + T::LDS_ALLOC - 16);
+  // two stages, the FP4 scale buffers (16 KB), 1 KB per wave for epilogue scales, the schedule's broadcast word
+  __shared__ __attribute__((aligned(16))) uint8_t lds[W4_LDS_BYTES];
+  int& s_bcast = *(int*)(lds + W4_LDS_BYTES - 16);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -276,6 +283,22 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   int nst = 0;             // 1: the previous tile's epilogue issued exactly 32 stores per wave (its fast path)
   uint32_t scbuf = 0;
   const int kh = p.k_iters >> 1;
+  // Fused epilogue: a full tile with bf16 output (and, for FP8, both scale vectors; for the other
+  // kinds, none) is not stored by the code below but by the NEXT tile's K loop, which reads each
+  // accumulator row block out just before its first K step overwrites it.  The last tile of a workgroup
+  // always takes the code below.  An FP8 K loop copies its own tile's scale vectors into LDS for that.
+  int fe = 0;                       // 1: the previous tile's sums are still in the accumulators
+  const uint8_t* cprev = (const uint8_t*)p.C;   // C[first row of the wave's quarter][its first column] of that tile
+  const bool fe_shape = p.c_line && !p.bias && p.c_type == DT_BF16 && p.c_sm < (1 << 26) && (p.debug & 4) == 0 &&
+                        ((T::DT == DT_FP8) == (p.sa != nullptr));
+  // a lane's C offset from cprev, the same in every row block (rows of a row block are c_sm apart);
+  // lane * 4; where the lane finds the scales of its rows 16 i + r and of its columns 32 q + 8 g + 0..7
+  v4i eo;
+  eo[0] = (int)(((uint32_t)ln.r * (uint32_t)p.c_sm + 8u * (uint32_t)ln.g) * 2u);
+  eo[1] = lane * 4;
+  eo[2] = (int)(lds0 + (uint32_t)W4_EPS_OFFSET + (uint32_t)wave * 1024u + (uint32_t)ln.r * 4u);
+  eo[3] = (int)(lds0 + (uint32_t)W4_EPS_OFFSET + (uint32_t)wave * 1024u + 512u + (uint32_t)ln.g * 32u);
+  const uint32_t s_cstep = uniform((uint32_t)p.c_sm * 32u);
   while (have) {
     // the tile after this one: its first two K steps are requested during this tile's last two.  With
     // none left the copies read this tile's first steps again; nobody uses them.
@@ -284,70 +307,83 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     W4TileArgs cur, nxt;
     w4_tile_args<T>(p, w.tc, ln, cur);
     w4_tile_args<T>(p, wnext.tc, ln, nxt);
-    v8i sc;
-    sc[0] = (int)(lds0 + 131072u + (uint32_t)(ln.wm0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
-    sc[1] = (int)(lds0 + 131072u + (uint32_t)(256 + ln.wn0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
-    sc[2] = (int)cur.sca; sc[3] = (int)cur.scb; sc[4] = (int)nxt.sca; sc[5] = (int)nxt.scb; sc[6] = 0; sc[7] = 0;
+    const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
+                      (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
+    const bool regs = T::DT == DT_FP8 && fast && p.sa;    // the K loop copies this tile's scale vectors
     const uint8_t *sA = uniform(cur.A), *sB = uniform(cur.B), *sAn = uniform(nxt.A), *sBn = uniform(nxt.B);
-    const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst);
+    const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst), s_fe = uniform(fe);
+    const uint8_t* s_cprev = uniform(cprev);
     scbuf = uniform(scbuf);
     if constexpr (T::DT == DT_FP8) {
+      // (a tile without scales or off the fast path loads 512 bytes of its operands instead; nobody uses them)
+      const uint8_t* s_sap = uniform(regs ? (const uint8_t*)(p.sa + w.tc.m0 + ln.wm0) : cur.A);
+      const uint8_t* s_sbp = uniform(regs ? (const uint8_t*)(w.tc.sb + w.tc.n0 + ln.wn0) : cur.B);
       asm volatile(
 #include "w4_kloop_fp8.inc"
           : [scbuf] "+s"(scbuf)
-          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
           :
-#include "w4_clobbers.inc"
+#include "w4_clobbers_fp8.inc"
       );
     } else if constexpr (T::DT == DT_BF16) {
       asm volatile(
 #include "w4_kloop_bf16.inc"
           : [scbuf] "+s"(scbuf)
-          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo)
           :
-#include "w4_clobbers.inc"
+#include "w4_clobbers_bf16.inc"
       );
     } else if constexpr (T::DT == DT_F16) {
       asm volatile(
 #include "w4_kloop_f16.inc"
           : [scbuf] "+s"(scbuf)
-          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo)
           :
-#include "w4_clobbers.inc"
+#include "w4_clobbers_f16.inc"
       );
     } else {
+      v8i sc;
+      sc[0] = (int)(lds0 + 131072u + (uint32_t)(ln.wm0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
+      sc[1] = (int)(lds0 + 131072u + (uint32_t)(256 + ln.wn0 + ln.r) * 16u + (uint32_t)ln.g * 2u);
+      sc[2] = (int)cur.sca; sc[3] = (int)cur.scb; sc[4] = (int)nxt.sca; sc[5] = (int)nxt.scb; sc[6] = eo[0]; sc[7] = 0;
       const uint8_t *sMa = uniform(cur.mxa), *sMb = uniform(cur.mxb), *sMan = uniform(nxt.mxa), *sMbn = uniform(nxt.mxb);
       asm volatile(
 #include "w4_kloop_fp4.inc"
           : [scbuf] "+s"(scbuf)
-          : [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [sc] "{v[232:239]}"(sc),
-            [A] "s"(sA), [B] "s"(sB), [An] "s"(sAn), [Bn] "s"(sBn), [mxa] "s"(sMa), [mxb] "s"(sMb),
-            [mxan] "s"(sMan), [mxbn] "s"(sMbn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst)
+          : W4_COMMON_OPERANDS, [sc] "{v[232:239]}"(sc), [mxa] "s"(sMa), [mxb] "s"(sMb), [mxan] "s"(sMan), [mxbn] "s"(sMbn)
           :
-#include "w4_clobbers.inc"
+#include "w4_clobbers_fp4.inc"
       );
     }
-    const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
-                      (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
-    // Every workgroup reaches its epilogue at about the same time, so C arrives as bursts of 32 MB; the
-    // L2s take such a burst as ordinary write-back lines and drain it behind the next K steps, while
-    // non-temporal stores go to the fabric at once and hold the waves at the store queue (measured:
-    // FP8 8192x28672x8192 1.24 -> 1.20 ms, MXFP4 8192x8192x16384 0.440 -> 0.415 ms without the hint).
+    if (fast && fe_shape && have_next) {
+      // stored by the next tile's K loop
+      fe = 1;
+      cprev = (const uint8_t*)p.C + ((int64_t)(w.tc.m0 + ln.wm0) * p.c_sm + (w.tc.n0 + ln.wn0)) * 2;
+      nst = 0;
+    } else {
+      fe = 0;
+      // Every workgroup reaches its epilogue at about the same time, so C arrives as bursts of 32 MB; the
+      // L2s take such a burst as ordinary write-back lines and drain it behind the next K steps, while
+      // non-temporal stores go to the fabric at once and hold the waves at the store queue (measured:
+      // FP8 8192x28672x8192 1.24 -> 1.20 ms, MXFP4 8192x8192x16384 0.440 -> 0.415 ms without the hint).
 #ifdef W4_LAB_NT
-    const bool c_nt = p.c_nt;
+      const bool c_nt = p.c_nt;
 #else
-    const bool c_nt = false;
+      const bool c_nt = false;
 #endif
-    if (fast) {
-      if (p.c_type == DT_BF16) { if (c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_BF16, false>(p, w.tc, ln); }
-      else { if (c_nt) epilogue_w4_fast<T, DT_F16, true>(p, w.tc, ln); else epilogue_w4_fast<T, DT_F16, false>(p, w.tc, ln); }
-    } else if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
-    else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
-    else epilogue_w4<T, DT_F32>(p, w.tc, ln);
-    nst = fast ? 1 : 0;
+      if (fast) {
+        if (p.c_type == DT_BF16) {
+          if (c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln);
+          else epilogue_w4_fast<T, DT_BF16, false>(p, w.tc, ln);
+        } else {
+          if (c_nt) epilogue_w4_fast<T, DT_F16, true>(p, w.tc, ln);
+          else epilogue_w4_fast<T, DT_F16, false>(p, w.tc, ln);
+        }
+      } else if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
+      else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
+      else epilogue_w4<T, DT_F32>(p, w.tc, ln);
+      nst = fast ? 1 : 0;
+    }
     w.tc = wnext.tc;
     have = have_next;
     first = 0;

@@ -2,85 +2,110 @@
 """Writes the hand-scheduled K loop of the 4-wave 256x256 tile kernels (gemm_w4.h) as inline-assembly text.
 
     python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: fp4, bf16, f16)
-    python3 gen_w4.py clobbers > w4_clobbers.inc
+    python3 gen_w4.py clobbers fp8 > w4_clobbers_fp8.inc
+    python3 gen_w4.py check                          (walks every kind through the wait-count checker)
 
 One workgroup = 4 waves (one per SIMD), wave (wm, wn) owns the 128x128 quarter of a 256x256 output
 tile: 8x8 MFMA tiles of 16x16, i.e. 256 accumulator registers a[0:255]; acc(i, j) of A row block i and
 B row block j sits in a[(8i+j)*4 .. +3].  A K step is 128 bytes of every operand row (128 FP8 values,
-256 FP4 values or 64 16-bit values); LDS holds two stages of 64 KB: stage s at s*65536, A rows at +0, B rows at +32768,
-row r at r*128 with its eight 16-byte chunks XOR-swizzled (the layout the 8-wave kernels use).  FP4
-adds two 8 KB buffers of E8M0 scales behind the stages (16 scale bytes per row = two K steps).
+256 FP4 values or 64 16-bit values); LDS holds two stages of 64 KB: stage s at s*65536, A rows at +0,
+B rows at +32768, row r at r*128 with its eight 16-byte chunks XOR-swizzled (the layout the 8-wave
+kernels use).  FP4 adds two 8 KB buffers of E8M0 scales behind the stages (16 scale bytes per row =
+two K steps).
 
-The text below is the code of ONE asm statement that runs the whole K loop of one output tile:
+The text is the code of ONE asm statement that runs the whole K loop of one output tile (at least four
+K steps, an even number):
 
   entry      (first tile of the workgroup only) copies of K steps 0 and 1 and of scale group 0
   per K step eight row blocks of MFMAs (row block i multiplies A fragment i with the eight B fragments);
-             the A fragment of row block i+3 is requested when row block i starts (four fragment
-             buffers), the B fragments of the next step sit in the other of two B register sets;
-             in front of row block 5 all LDS reads of the step have been issued:
-             lgkmcnt(0), vmcnt(0) (next step's copies have landed), s_barrier, and behind it, between
-             the 24 MFMAs of row blocks 5..7, the copies of step +2 into the stage just freed and the
-             reads of the next step's B fragments, scales and first A fragments
+             A fragments go through four buffers, the B fragments of the next step sit in the other of
+             two register sets.  Two sync points (wait + s_barrier) per step, each followed by copies of
+             step +2 into LDS that every wave has just declared free:
+               X, in row block 1: this step's B fragments and A fragments 0..3 are in registers -> the
+                  B half of the stage and the A rows of row blocks 0..3 ("A lo") take step +2; it also
+                  publishes "A hi" (row blocks 4..7) of THIS step, which is read from here on;
+               Y, in row block 5: A fragments 4..7 are in registers -> "A hi" takes step +2; it
+                  publishes B and "A lo" of the NEXT step for the reads that follow.
+             Every copy is waited for one and a half K steps after it was issued and two to three
+             bursts overlap in time (one burst per step that must land within one step leaves the
+             L2 -> LDS path idle for the latency of its first byte and then stalls the MFMAs).
+  first two  the MFMAs of step 0 start from zero (no clearing pass).  When the caller says so (%[fe]) the
+  K steps    accumulators still hold the PREVIOUS tile's sums: each row block is then read out, scaled,
+             rounded to bf16 and stored just before step 0 overwrites it, between the MFMAs of the row
+             block before -- the epilogue costs no MFMA-idle time and its stores are spread over a K step.
+             Step 1 loads this tile's own epilogue scales (FP8) into registers that the caller carries
+             to the next call.
   last two   the copies go to the NEXT tile's first two K steps (the caller passes the next tile's
   K steps    addresses, or the same tile's again when there is none), so the copy pipeline never drains
              between tiles; no fragments are prefetched across the tile boundary.
 
-K must be a multiple of two K steps (the loop body is the even step followed by the odd step).
+vmcnt counts vector-memory operations in issue order, loads and stores alike, so every wait names how
+many YOUNGER operations may still be in flight.  Those numbers depend on what ran before (the entry's
+copies, a previous tile's epilogue stores issued by compiled code, the fused epilogue's own stores);
+`check` replays the instruction stream of every such history and proves each wait at least as strict
+as needed.
 
-Register map (VGPR):  0..127  B fragment sets 0/1 (8 fragments x 8 registers each)
+Register map (VGPR):  0..127   B fragment sets 0/1 (8 fragments x 8 registers each)
                       128..159 A fragment buffers 0..3
-                      160..191 FP4 scale registers, set p: A rows 160+16p+i, B rows 168+16p+j
-                      192..207 inputs: byte offsets of this tile's copies (A 192+i, B 200+i, i = copy instruction)
-                      208..223 inputs: the same for the next tile
-                      224..231 inputs: fragment read addresses (A lo, A hi, B lo, B hi) for stage 0, then stage 1
-                      232..237 inputs: scale read addresses (A, B), scale copy offsets (A, B) now and next
-                      240, 241 scratch: scale read addresses of the current scale buffer
-SGPR 70..82 are scratch (copy cursors, loop counter, scale buffer toggle, first-step flag).
+                      160..191 FP4: E8M0 scale registers (set p: A rows 160+16p+i, B rows 168+16p+j);
+                               FP8: epilogue column scales sb (in/out)
+                      192..207 in: byte offsets of this tile's copies (A 192+i, B 200+i, i = copy instruction)
+                      208..223 in: the same for the next tile
+                      224..231 in: fragment read addresses (A lo, A hi, B lo, B hi) for stage 0, then stage 1
+                      FP4:  232..237 in: scale read addresses (A, B), scale copy offsets (A, B) now and next;
+                            238 in: C offset of this lane; 240, 241 scale read addresses of the current buffer
+                      else: 240 in: C offset of this lane; FP8: 241 in: lane * 4, 242 in / 243 in: LDS
+                            addresses this lane reads its row / column scales from
+                      The fused epilogue works in B fragment set 1 (64..127), which is free from the end of
+                      the previous tile until the second half of step 0: column scales 64..95, row scales
+                      96..103, scratch 104..113.
+SGPR 70..89 are scratch (copy cursors, loop counter, scale buffer toggle, flags, C row pointer).
 """
+import os
 import sys
 
 STAGE = 65536
 BOFF = 32768
 SC0 = 131072          # scale buffers behind the two stages
 SCBUF = 8192
-NST = 32              # stores per wave of the fast epilogue (256x256 16-bit values, 16 bytes per lane and store)
-import os
-BND = int(os.environ.get("W4GEN_BND", "5"))   # the K-step boundary sits in front of this row block
+EPS = SC0 + 2 * SCBUF  # epilogue scales: 1 KB per wave
+NST = 32              # stores per wave of an epilogue (256x256 16-bit values, 16 bytes per lane and store)
 
-S_CA, S_CB, S_CSA, S_CSB, S_CNT, S_SCN, S_T, S_SCIN, S_FIRST = 70, 72, 74, 76, 78, 79, 80, 81, 82
+S_CA, S_CB, S_CSA, S_CSB, S_CNT, S_SCN, S_T, S_SCIN, S_AFTER, S_CROW, S_T2 = 70, 72, 74, 76, 78, 79, 80, 81, 82, 84, 86
+
+
+class Op:
+    """one instruction; vm: tag of the group of vector-memory operations it belongs to (None: not one)"""
+    def __init__(self, text, vm=None):
+        self.text, self.vm = text, vm
+
+
+class WaitVm:
+    """s_waitcnt vmcnt(n): everything up to and including group `awaits` must have completed.  vals maps
+    a history ("a" first tile of the workgroup, "b" previous tile's epilogue = 32 compiled stores, "c" =
+    unknown compiled stores, "d" fused epilogue, "s" steady state, "f" first even step after the first
+    two) to n."""
+    def __init__(self, awaits, vals):
+        self.awaits, self.vals = awaits, {k: min(63, v) for k, v in vals.items()}
 
 
 class Gen:
-    def __init__(self, kind, dma_every=1, lab=()):
+    def __init__(self, kind, lab=()):
         self.kind = kind                # "fp8" | "fp4" | "bf16" | "f16"
         self.fp4 = kind == "fp4"        # (the only kind with E8M0 scale operands)
-        self.out = []
+        self.scaled_epi = kind == "fp8"  # the fused epilogue multiplies by sa[m] * sb[n]
         self.nm = 8 if kind == "fp8" else 16      # MFMAs per row block (FP8: one of K = 128 per fragment pair; others: two half-K ones)
-        self.dma_every = dma_every
+        self.nsc = 4 if self.scaled_epi else 0    # copies of the tile's own epilogue scales (step 1)
         self.lbl = 0
         # how far (in MFMAs) into row blocks 1 and 5 the two sync points of a K step sit
         self.xoff = int(os.environ.get("W4GEN_XOFF", str(self.nm // 2)))
         self.yoff = int(os.environ.get("W4GEN_YOFF", str(self.nm // 2)))
-        # measurement builds (W4GEN_LAB=nomfma,nodma,noread,nobar): leave one kind of instruction out to time
-        # the rest; results are then meaningless
+        # measurement builds (W4GEN_LAB=nomfma,nodma,noread,nobar,novm,nolgk): leave one kind of
+        # instruction out to time the rest; results are then meaningless
         self.lab = set(lab)
-
-    def e(self, s):
-        if "nomfma" in self.lab and s.startswith("v_mfma"):
-            return
-        if "nodma" in self.lab and s.startswith("global_load_lds"):
-            return
-        if "noread" in self.lab and s.startswith("ds_read"):
-            return
-        if "nobar" in self.lab and s.startswith("s_barrier"):
-            return
-        if "novm" in self.lab and s.startswith("s_waitcnt vmcnt"):
-            return
-        if "nolgk0" in self.lab and s == "s_waitcnt lgkmcnt(0)":
-            return
-        if "nolgk" in self.lab and s.startswith("s_waitcnt lgkmcnt"):
-            return
-        self.out.append(s)
+        self.v_coff = 238 if self.fp4 else 240
+        self.v_lane4, self.v_sa_rd, self.v_sb_rd = 241, 242, 243
+        self.v_sb, self.v_sa, self.epi_tmp = 64, 96, 104
 
     # ---- register names ---------------------------------------------------------------------------
     @staticmethod
@@ -106,112 +131,181 @@ class Gen:
     # ---- building blocks --------------------------------------------------------------------------
     def frag_read(self, dst, op, stage, t):
         """both 16-byte halves of fragment t (16 rows x 128 bytes of K) of operand op"""
-        return [f"ds_read_b128 v[{dst}:{dst + 3}], v{self.fa(op, 0, stage)} offset:{t * 2048}",
-                f"ds_read_b128 v[{dst + 4}:{dst + 7}], v{self.fa(op, 1, stage)} offset:{t * 2048}"]
+        return [Op(f"ds_read_b128 v[{dst}:{dst + 3}], v{self.fa(op, 0, stage)} offset:{t * 2048}"),
+                Op(f"ds_read_b128 v[{dst + 4}:{dst + 7}], v{self.fa(op, 1, stage)} offset:{t * 2048}")]
 
     def scale_reads(self, p, half):
         """E8M0 bytes of one K step for all row blocks: two bytes (k slices 0, 1) per lane and row block"""
         r = []
         for i in range(8):
-            r.append(f"ds_read_u16 v{self.scA(p, i)}, v240 offset:{i * 256 + half * 8}")
+            r.append(Op(f"ds_read_u16 v{self.scA(p, i)}, v240 offset:{i * 256 + half * 8}"))
         for j in range(8):
-            r.append(f"ds_read_u16 v{self.scB(p, j)}, v241 offset:{j * 256 + half * 8}")
+            r.append(Op(f"ds_read_u16 v{self.scB(p, j)}, v241 offset:{j * 256 + half * 8}"))
         return r
 
-    def dma(self, stage, nxt):
+    def dma(self, stage, nxt, tag):
         """the 16 LDS-direct copies of one K step (A then B), each as [m0 setup, wait state, load]"""
         ops = []
         base = 208 if nxt else 192
         for op, cur in ((0, S_CA), (1, S_CB)):
             for i in range(8):
                 imm = stage * STAGE + op * BOFF + i * 4096
-                ops.append([f"s_add_u32 m0, %[wl], {imm}", "s_nop 0",
-                            f"global_load_lds_dwordx4 v{base + op * 8 + i}, s[{cur}:{cur + 1}]"])
+                ops.append([Op(f"s_add_u32 m0, %[wl], {imm}"), Op("s_nop 0"),
+                            Op(f"global_load_lds_dwordx4 v{base + op * 8 + i}, s[{cur}:{cur + 1}]", tag)])
         return ops
 
     def dma_advance(self):
-        return [f"s_add_u32 s{S_CA}, s{S_CA}, 128", f"s_addc_u32 s{S_CA + 1}, s{S_CA + 1}, 0",
-                f"s_add_u32 s{S_CB}, s{S_CB}, 128", f"s_addc_u32 s{S_CB + 1}, s{S_CB + 1}, 0"]
+        return [Op(f"s_add_u32 s{S_CA}, s{S_CA}, 128"), Op(f"s_addc_u32 s{S_CA + 1}, s{S_CA + 1}, 0"),
+                Op(f"s_add_u32 s{S_CB}, s{S_CB}, 128"), Op(f"s_addc_u32 s{S_CB + 1}, s{S_CB + 1}, 0")]
 
-    def scale_dma(self, nxt):
+    def scale_dma(self, nxt, tag):
         """copy of one scale group (16 bytes per row, A rows then B rows) into the buffer s79 names, then toggle it"""
         va, vb = (236, 237) if nxt else (234, 235)
-        return [[f"s_add_u32 s{S_T}, %[wl], s{S_SCN}", f"s_add_u32 m0, s{S_T}, {SC0}", "s_nop 0",
-                 f"global_load_lds_dwordx4 v{va}, s[{S_CSA}:{S_CSA + 1}]"],
-                [f"s_add_u32 m0, s{S_T}, {SC0 + 4096}", "s_nop 0",
-                 f"global_load_lds_dwordx4 v{vb}, s[{S_CSB}:{S_CSB + 1}]",
-                 f"s_xor_b32 s{S_SCN}, s{S_SCN}, {SCBUF}",
-                 f"s_add_u32 s{S_CSA}, s{S_CSA}, 16", f"s_addc_u32 s{S_CSA + 1}, s{S_CSA + 1}, 0",
-                 f"s_add_u32 s{S_CSB}, s{S_CSB}, 16", f"s_addc_u32 s{S_CSB + 1}, s{S_CSB + 1}, 0"]]
+        return [[Op(f"s_add_u32 s{S_T}, %[wl], s{S_SCN}"), Op(f"s_add_u32 m0, s{S_T}, {SC0}"), Op("s_nop 0"),
+                 Op(f"global_load_lds_dwordx4 v{va}, s[{S_CSA}:{S_CSA + 1}]", tag)],
+                [Op(f"s_add_u32 m0, s{S_T}, {SC0 + 4096}"), Op("s_nop 0"),
+                 Op(f"global_load_lds_dwordx4 v{vb}, s[{S_CSB}:{S_CSB + 1}]", tag),
+                 Op(f"s_xor_b32 s{S_SCN}, s{S_SCN}, {SCBUF}"),
+                 Op(f"s_add_u32 s{S_CSA}, s{S_CSA}, 16"), Op(f"s_addc_u32 s{S_CSA + 1}, s{S_CSA + 1}, 0"),
+                 Op(f"s_add_u32 s{S_CSB}, s{S_CSB}, 16"), Op(f"s_addc_u32 s{S_CSB + 1}, s{S_CSB + 1}, 0")]]
 
-    def mfma(self, p, i, slot):
-        """MFMA number `slot` of row block i: B fragment first (its rows become the output rows a lane holds)"""
+    def mfma(self, p, i, slot, zero):
+        """MFMA number `slot` of row block i: B fragment first (its rows become the output rows a lane
+        holds).  zero: first K step of a tile, the sum starts from 0 instead of the accumulator."""
         if self.kind == "fp8":
             j = slot
             acc = (i * 8 + j) * 4
             b, a = self.vB(p, j), self.vA(i)
-            return f"v_mfma_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 7}], v[{a}:{a + 7}], a[{acc}:{acc + 3}]"
+            c = "0" if zero else f"a[{acc}:{acc + 3}]"
+            return Op(f"v_mfma_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 7}], v[{a}:{a + 7}], {c}")
         # two MFMAs per accumulator and K step, k slice outermost so that the same accumulator comes up
         # again only eight instructions later
         ks, j = slot // 8, slot % 8
         acc = (i * 8 + j) * 4
         b, a = self.vB(p, j) + 4 * ks, self.vA(i) + 4 * ks
+        c = "0" if (zero and ks == 0) else f"a[{acc}:{acc + 3}]"
         if self.kind in ("bf16", "f16"):
-            return f"v_mfma_f32_16x16x32_{self.kind} a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], a[{acc}:{acc + 3}]"
-        return (f"v_mfma_scale_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], a[{acc}:{acc + 3}], "
-                f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
+            return Op(f"v_mfma_f32_16x16x32_{self.kind} a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}")
+        return Op(f"v_mfma_scale_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}, "
+                  f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
+
+    def epilogue_block(self, i, tag):
+        """The previous tile's row block i: for each of its four column groups read eight sums, scale
+        (FP8: acc * (sa[m] * sb[n]), the order the compiled epilogues use), round to bf16 pairs, store 16
+        bytes.  Returns the instructions in order; the row pointer s[84:85] moves on afterwards."""
+        t = self.epi_tmp
+        e = [t, t + 1, t + 2, t + 3]
+        s, pk = t + 4, [t + 6, t + 7, t + 8, t + 9]     # (register tuples start at even registers)
+        out = []
+        for q in range(4):
+            for h in range(2):
+                base = (i * 8 + 2 * q + h) * 4
+                for x in range(4):
+                    out.append(Op(f"v_accvgpr_read_b32 v{e[x]}, a{base + x}"))
+                if self.scaled_epi:
+                    for x in range(4):
+                        out.append(Op(f"v_mul_f32 v{s}, v{self.v_sa + i}, v{self.v_sb + q * 8 + h * 4 + x}"))
+                        out.append(Op(f"v_mul_f32 v{e[x]}, v{e[x]}, v{s}"))
+                out.append(Op(f"v_cvt_pk_bf16_f32 v{pk[2 * h]}, v{e[0]}, v{e[1]}"))
+                out.append(Op(f"v_cvt_pk_bf16_f32 v{pk[2 * h + 1]}, v{e[2]}, v{e[3]}"))
+            out.append(Op(f"global_store_dwordx4 v{self.v_coff}, v[{pk[0]}:{pk[3]}], s[{S_CROW}:{S_CROW + 1}] offset:{q * 64}", tag))
+        out.append(Op(f"s_add_u32 s{S_CROW}, s{S_CROW}, %[cstep]"))
+        out.append(Op(f"s_addc_u32 s{S_CROW + 1}, s{S_CROW + 1}, 0"))
+        return out
+
+    def scale_loads(self, tag):
+        """This tile's own epilogue scales (sa of the wave's 128 rows, sb of its 128 columns: 2 x 512 bytes)
+        go to the wave's 1 KB of LDS behind the stages; the tile that runs the epilogue reads them there."""
+        out = [Op(f"s_mov_b64 s[{S_T2}:{S_T2 + 1}], %[sap]")]
+        for n, (base, half) in enumerate((("sap", 0), ("sap", 1), ("sbp", 0), ("sbp", 1))):
+            if half == 0:
+                out.append(Op(f"s_mov_b64 s[{S_T2}:{S_T2 + 1}], %[{base}]"))
+            else:
+                out += [Op(f"s_add_u32 s{S_T2}, s{S_T2}, 256"), Op(f"s_addc_u32 s{S_T2 + 1}, s{S_T2 + 1}, 0")]
+            out += [Op(f"s_add_u32 m0, %[wl], {EPS + n * 256}"), Op("s_nop 0"),
+                    Op(f"global_load_lds_dword v{self.v_lane4}, s[{S_T2}:{S_T2 + 1}]", tag)]
+        return out[1:]
+
+    def scale_reads_epi(self):
+        """the previous tile's scales of this lane: rows 16 i + r, columns 32 q + 8 g + 0..7"""
+        out = []
+        for i in range(8):
+            out.append(Op(f"ds_read_b32 v{self.v_sa + i}, v{self.v_sa_rd} offset:{i * 64}"))
+        for q in range(4):
+            for h in range(2):
+                r = self.v_sb + q * 8 + h * 4
+                out.append(Op(f"ds_read_b128 v[{r}:{r + 3}], v{self.v_sb_rd} offset:{q * 128 + h * 16}"))
+        return out
 
     # ---- one K step -------------------------------------------------------------------------------
-    def wait_vm(self, n, n_stores, n_cons):
-        """s_waitcnt vmcnt(n) in the steady state.  While s82 is set (first K steps of a tile) the previous
-        tile's epilogue stores are younger than the copies waited for: with %[nst] they are exactly 32 per
-        wave and the wait allows for them (n_stores), otherwise it assumes none (n_cons)."""
-        self.lbl += 1
-        f, g, d = (f"W4_V{x}{self.lbl}_%=" for x in "FGD")
-        return [f"s_cmp_lg_u32 s{S_FIRST}, 0", f"s_cbranch_scc1 {f}", f"s_waitcnt vmcnt({n})", f"s_branch {d}",
-                f"{f}:", "s_cmp_lg_u32 %[nst], 0", f"s_cbranch_scc1 {g}", f"s_waitcnt vmcnt({n_cons})", f"s_branch {d}",
-                f"{g}:", f"s_waitcnt vmcnt({n_stores})", f"{d}:"]
-
-    def step(self, p, nxt, prefetch):
+    def step(self, p, nxt, prefetch, flavor="steady"):
         """K step in stage p (= B set p, scale set p).  nxt: the copies issued in this step read the
-        next tile.  prefetch: request the following step's fragments in the tail.
-
-        Two sync points (wait + s_barrier) per step, each followed by copies of step +2 into LDS that
-        every wave has just declared free:
-          X, in front of row block 1: this step's B fragments and A fragments 0..3 are in registers
-             -> B half of the stage and the A rows of row blocks 0..3 ("A lo") take step +2;
-             it also publishes "A hi" of THIS step (row blocks 4..7), which is read from here on;
-          Y, in front of row block 5 (the step boundary): A fragments 4..7 are in registers
-             -> "A hi" takes step +2; it publishes B and "A lo" of the NEXT step for the tail's reads.
-        Every copy is therefore waited for one and a half K steps after it was issued, and two to
-        three bursts overlap in time: one burst per step that has to land within one step leaves the
-        L2 -> LDS path idle for the latency of its first byte and then stalls the MFMAs at the wait.
-        vmcnt counts in issue order, so each wait names how many younger copies may stay in flight."""
+        next tile.  prefetch: request the following step's fragments at the end.  flavor: "steady",
+        "first0" (step 0 of a tile), "first0_fe" (with the previous tile's epilogue fused in), "first1".
+        Group tags are relative to this step: ("X", 0), ("Y", 0), awaited ("Y", -2), ("X", -1)."""
         nm = self.nm
         total = 8 * nm
-        self.e(f"; ---- K step, stage {p}{' (copies: next tile)' if nxt else ''}{'' if prefetch else ' (last of the tile)'}")
+        first0 = flavor in ("first0", "first0_fe")
+        fe = flavor == "first0_fe"
+        out = [Op(f"; ---- K step, stage {p}, {flavor}{' (copies: next tile)' if nxt else ''}{'' if prefetch else ' (last of the tile)'}")]
         pre = [[] for _ in range(total)]      # in front of MFMA slot m
         post = [[] for _ in range(total)]     # behind it
-        ops = self.dma(p, nxt)
+        ops = self.dma(p, nxt, None)
         lo = [ops[i] for i in (0, 1, 4, 5)]                 # A rows of row blocks 0..3 (both wave rows)
         hi = [ops[i] for i in (2, 3, 6, 7)]
         ops_b = ops[8:]
+        for o in lo + ops_b:
+            o[-1].vm = ("X", 0)
+        for o in hi:
+            o[-1].vm = ("Y", 0)
         adv = self.dma_advance()
         adv_a, adv_b = adv[:2], adv[2:]
-        sc = self.scale_dma(nxt) if (self.fp4 and p == 0) else []
-        nx = len(ops_b) + len(lo) + len(sc)                # copies issued behind X of this step
-        nx_other = 12 + (2 if (self.fp4 and p == 1) else 0)   # ... behind X of the neighbouring steps
+        sc = self.scale_dma(nxt, ("X", 0)) if (self.fp4 and p == 0) else []
+        nx = len(ops_b) + len(lo) + len(sc)                   # copies issued behind X of this step
+        nxo = 12 + (2 if (self.fp4 and p == 1) else 0)        # ... behind X of the neighbouring steps
+        nsc = self.nsc
+        # fused epilogue: row block 0 in front of the first MFMA, row block i+1 between the MFMAs of row block i
+        n_st = [0] * (total + 1)   # stores issued in front of slot m
+        if fe:
+            # row block 0 in front of the first MFMA, the others spread over row blocks 0..4: block k is
+            # done before slot 5 nm k / 7 <= nm k, where its accumulators are overwritten, and everything
+            # is done before the fragments of step 1 arrive in the registers used here
+            blocks = [self.epilogue_block(i, ("ST", 0)) for i in range(8)]
+            pre[0] += [Op("s_waitcnt lgkmcnt(15)")] if self.scaled_epi else []
+            pre[0] += blocks[0]
+            rest = [o for b in blocks[1:] for o in b]
+            for n, o in enumerate(rest):
+                post[n * 5 * nm // len(rest)].append(o)
         # row block 0
+        if flavor == "first1" and nsc:
+            pre[0] += self.scale_loads(("SC", 0))
         pre[0] += self.frag_read(self.vA(3), 0, p, 3)
-        pre[0].append("s_waitcnt lgkmcnt(6)")
-        # X: part of the way into row block 1, so that the read of A fragment 3 (requested when row block 0
-        # started) has had time to return before lgkmcnt(0) asks for it
+        pre[0].append(Op("s_waitcnt lgkmcnt(6)"))
         xs = nm + self.xoff
-        # (X of step 0: nothing of this tile may be assumed younger than the stores; X of step 1: the
-        # steady-state count already demands that the stores are done)
-        pre[xs] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx_other + 4, nx_other + 4 + NST, 0 if p == 0 else nx_other + 4) + ["s_barrier"]
-        if p == 1:
-            post[xs].append(f"s_mov_b32 s{S_FIRST}, 0")
+        tail0 = 5 * nm + self.yoff
+        if fe:
+            # (stores in program order in front of X and Y)
+            def stores_before(slot):
+                c = sum(1 for o in pre[0] if o.vm == ("ST", 0))
+                for m in range(slot):
+                    c += sum(1 for o in post[m] if o.vm == ("ST", 0))
+                return c
+            sx, sy = stores_before(xs), stores_before(tail0)
+        # X
+        if flavor == "steady":
+            if p == 0 and nsc:
+                wx = WaitVm(("Y", -2), {"s": nxo + 4, "f": nxo + 4 + nsc})
+            else:
+                wx = WaitVm(("Y", -2), {"s": nxo + 4})
+        elif flavor == "first0":
+            wx = WaitVm(("Y", -2), {"a": nxo + 4, "b": nxo + 4 + NST, "c": 0})
+        elif flavor == "first0_fe":
+            wx = WaitVm(("Y", -2), {"d": nxo + 4 + sx})
+        else:   # first1: the previous tile's stores (compiled or fused) are younger than the awaited copies
+            wx = WaitVm(("Y", -2), {"a": nxo + 4 + nsc, "b": nxo + 4 + nsc + NST, "c": nxo + 4 + nsc, "d": nxo + 4 + nsc + NST})
+        pre[xs] += [Op("s_waitcnt lgkmcnt(0)"), wx, Op("s_barrier")]
+        if flavor == "steady" and p == 0 and nsc:
+            post[xs].append(Op(f"s_mov_b32 s{S_AFTER}, 0"))
         pre[xs] += self.frag_read(self.vA(4), 0, p, 4)
         xops = ops_b + lo + sc
         span = 5 * nm - 2 - xs
@@ -222,20 +316,24 @@ class Gen:
         pre[3 * nm] += self.frag_read(self.vA(6), 0, p, 6)
         pre[4 * nm] += self.frag_read(self.vA(7), 0, p, 7)
         # (A fragment 4 was requested at X; fragments 5, 6, 7 are younger)
-        pre[4 * nm].append("s_waitcnt lgkmcnt(6)")
+        pre[4 * nm].append(Op("s_waitcnt lgkmcnt(6)"))
         # Y
-        tail0 = BND * nm + self.yoff
-        if p == 0:
-            pre[tail0] += ["s_waitcnt lgkmcnt(0)"] + self.wait_vm(nx + 4, nx + 4 + NST, nx) + ["s_barrier"]
-        else:
-            pre[tail0] += ["s_waitcnt lgkmcnt(0)", f"s_waitcnt vmcnt({nx + 4})", "s_barrier"]
+        if flavor == "steady":
+            wy = WaitVm(("X", -1), {"s": nx + 4})
+        elif flavor == "first0":
+            wy = WaitVm(("X", -1), {"a": nx + 4, "b": nx + 4 + NST, "c": nx})
+        elif flavor == "first0_fe":
+            wy = WaitVm(("X", -1), {"d": nx + 4 + sy})
+        else:   # first1: X of step 0 is awaited; a fused epilogue issued part of its stores behind that
+            wy = WaitVm(("X", -1), {"a": nx + 4 + nsc, "b": nx + 4 + nsc, "c": nx + 4 + nsc, "d": nx + 4 + nsc})
+        pre[tail0] += [Op("s_waitcnt lgkmcnt(0)"), wy, Op("s_barrier")]
         tail = total - tail0
         q = p ^ 1
         if prefetch:
             lds = []
             if self.fp4 and p == 1:
                 # the next step opens a new scale group: it sits in the other buffer
-                post[tail0] += [f"v_xor_b32 v240, {SCBUF}, v240", f"v_xor_b32 v241, {SCBUF}, v241"]
+                post[tail0] += [Op(f"v_xor_b32 v240, {SCBUF}, v240"), Op(f"v_xor_b32 v241, {SCBUF}, v241")]
             for j in range(8):
                 lds += self.frag_read(self.vB(q, j), 1, q, j)
             if self.fp4:
@@ -253,102 +351,207 @@ class Gen:
             post[tail0 + n * (tail - 2) // len(hi)] += op
         post[total - 2] += adv_a
         for m in range(total):
-            for l in pre[m]:
-                self.e(l)
-            self.e(self.mfma(p, m // nm, m % nm))
-            for l in post[m]:
-                self.e(l)
+            out += pre[m]
+            out.append(self.mfma(p, m // nm, m % nm, first0))
+            out += post[m]
+        return out
 
     # ---- the whole K loop of one tile -------------------------------------------------------------------
-    def kloop(self):
-        e = self.e
-        fp4 = self.fp4
-        e("; ==== 4-wave 256x256 K loop ====")
-        e(f"s_mov_b64 s[{S_CA}:{S_CA + 1}], %[A]")
-        e(f"s_mov_b64 s[{S_CB}:{S_CB + 1}], %[B]")
-        if fp4:
-            e(f"s_mov_b64 s[{S_CSA}:{S_CSA + 1}], %[mxa]")
-            e(f"s_mov_b64 s[{S_CSB}:{S_CSB + 1}], %[mxb]")
-            e(f"s_mov_b32 s{S_SCIN}, %[scbuf]")
-            e(f"s_mov_b32 s{S_SCN}, %[scbuf]")
-        e("s_cmp_eq_u32 %[first], 0")
-        e("s_cbranch_scc1 W4_RESUME%=")
-        # first tile of the workgroup: fill both stages (and the first scale group)
-        if fp4:
-            for op in self.scale_dma(False):
-                for l in op:
-                    e(l)
-        for st in (0, 1):
-            ops = self.dma(st, False)
-            for n in (8, 9, 10, 11, 12, 13, 14, 15, 0, 1, 4, 5, 2, 3, 6, 7):   # B, A lo, A hi: the order the steps use
-                for l in ops[n]:
-                    e(l)
-            for l in self.dma_advance():
-                e(l)
-        e("s_waitcnt vmcnt(16)")
-        e("s_barrier")
-        e("s_branch W4_ENTRY%=")
-        e("W4_RESUME%=:")
-        # later tiles: steps 0 and 1 (and scale group 0) were requested during the previous tile
-        e(f"s_add_u32 s{S_CA}, s{S_CA}, 256")
-        e(f"s_addc_u32 s{S_CA + 1}, s{S_CA + 1}, 0")
-        e(f"s_add_u32 s{S_CB}, s{S_CB}, 256")
-        e(f"s_addc_u32 s{S_CB + 1}, s{S_CB + 1}, 0")
-        if fp4:
-            e(f"s_add_u32 s{S_CSA}, s{S_CSA}, 16")
-            e(f"s_addc_u32 s{S_CSA + 1}, s{S_CSA + 1}, 0")
-            e(f"s_add_u32 s{S_CSB}, s{S_CSB}, 16")
-            e(f"s_addc_u32 s{S_CSB + 1}, s{S_CSB + 1}, 0")
-            e(f"s_xor_b32 s{S_SCN}, s{S_SCN}, {SCBUF}")
-        e("W4_ENTRY%=:")
-        e(f"s_mov_b32 s{S_FIRST}, 1")
-        # (either way s79 now names the buffer the NEXT scale group goes to)
-        if fp4:
-            e(f"v_add_u32 v240, s{S_SCIN}, v232")
-            e(f"v_add_u32 v241, s{S_SCIN}, v233")
+    def prologue(self):
+        out = []
+        if self.fp4:
+            for op in self.scale_dma(False, ("Y", -2)):
+                out += op
+        for st, tags in ((0, (("Y", -2), ("Y", -2), ("Y", -2))), (1, (("X", -1), ("X", -1), ("Y", -1)))):
+            ops = self.dma(st, False, None)
+            for grp, idx in zip(tags, ((8, 9, 10, 11, 12, 13, 14, 15), (0, 1, 4, 5), (2, 3, 6, 7))):   # B, A lo, A hi: the order the steps use
+                for n in idx:
+                    ops[n][-1].vm = grp
+                    out += ops[n]
+            out += self.dma_advance()
+        out += [WaitVm(("Y", -2), {"a": 16}), Op("s_barrier")]
+        return out
+
+    def entry_reads(self):
+        out = []
+        if self.fp4:
+            out += [Op(f"v_add_u32 v240, s{S_SCIN}, v232"), Op(f"v_add_u32 v241, s{S_SCIN}, v233")]
         for j in range(8):
-            for l in self.frag_read(self.vB(0, j), 1, 0, j):
-                e(l)
-        if fp4:
-            for l in self.scale_reads(0, 0):
-                e(l)
+            out += self.frag_read(self.vB(0, j), 1, 0, j)
+        if self.fp4:
+            out += self.scale_reads(0, 0)
         for t in range(3):
-            for l in self.frag_read(self.vA(t), 0, 0, t):
-                e(l)
-        for n in range(256):
-            e(f"v_accvgpr_write_b32 a{n}, 0")
-        e(f"s_sub_u32 s{S_CNT}, %[kh], 1")
-        e(f"s_cmp_eq_u32 s{S_CNT}, 0")
-        e("s_cbranch_scc1 W4_LAST%=")
-        e("W4_LOOP%=:")
-        self.step(0, False, True)
-        self.step(1, False, True)
-        e(f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1")
-        e(f"s_cmp_lg_u32 s{S_CNT}, 0")
-        e("s_cbranch_scc1 W4_LOOP%=")
-        e("W4_LAST%=:")
-        # the copy cursors move on to the next tile
-        e(f"s_mov_b64 s[{S_CA}:{S_CA + 1}], %[An]")
-        e(f"s_mov_b64 s[{S_CB}:{S_CB + 1}], %[Bn]")
+            out += self.frag_read(self.vA(t), 0, 0, t)
+        return out
+
+    def parts(self):
+        """the pieces of the program, each a list of Op / WaitVm"""
+        fp4 = self.fp4
+        P = {}
+        setup = [Op("; ==== 4-wave 256x256 K loop ===="),
+                 Op(f"s_mov_b64 s[{S_CA}:{S_CA + 1}], %[A]"), Op(f"s_mov_b64 s[{S_CB}:{S_CB + 1}], %[B]"),
+                 Op(f"s_mov_b64 s[{S_CROW}:{S_CROW + 1}], %[cprev]")]
         if fp4:
-            e(f"s_mov_b64 s[{S_CSA}:{S_CSA + 1}], %[mxan]")
-            e(f"s_mov_b64 s[{S_CSB}:{S_CSB + 1}], %[mxbn]")
-        self.step(0, True, True)
-        self.step(1, True, False)
+            setup += [Op(f"s_mov_b64 s[{S_CSA}:{S_CSA + 1}], %[mxa]"), Op(f"s_mov_b64 s[{S_CSB}:{S_CSB + 1}], %[mxb]"),
+                      Op(f"s_mov_b32 s{S_SCIN}, %[scbuf]"), Op(f"s_mov_b32 s{S_SCN}, %[scbuf]")]
+        P["setup"] = setup
+        P["prologue"] = self.prologue()
+        # later tiles: steps 0 and 1 (and scale group 0) were requested during the previous tile
+        resume = [Op(f"s_add_u32 s{S_CA}, s{S_CA}, 256"), Op(f"s_addc_u32 s{S_CA + 1}, s{S_CA + 1}, 0"),
+                  Op(f"s_add_u32 s{S_CB}, s{S_CB}, 256"), Op(f"s_addc_u32 s{S_CB + 1}, s{S_CB + 1}, 0")]
+        if fp4:
+            resume += [Op(f"s_add_u32 s{S_CSA}, s{S_CSA}, 16"), Op(f"s_addc_u32 s{S_CSA + 1}, s{S_CSA + 1}, 0"),
+                       Op(f"s_add_u32 s{S_CSB}, s{S_CSB}, 16"), Op(f"s_addc_u32 s{S_CSB + 1}, s{S_CSB + 1}, 0"),
+                       Op(f"s_xor_b32 s{S_SCN}, s{S_SCN}, {SCBUF}")]
+        P["resume"] = resume
+        # (either way s79 now names the buffer the NEXT scale group goes to)
+        P["entry_fe"] = self.scale_reads_epi() if self.scaled_epi else []
+        P["entry"] = [Op(f"s_mov_b32 s{S_AFTER}, 1")] + self.entry_reads()
+        P["first0"] = self.step(0, False, True, "first0")
+        P["first0_fe"] = self.step(0, False, True, "first0_fe")
+        P["first1"] = self.step(1, False, True, "first1")
+        P["steady0"] = self.step(0, False, True)
+        P["steady1"] = self.step(1, False, True)
+        # the copy cursors move on to the next tile
+        last_pre = [Op(f"s_mov_b64 s[{S_CA}:{S_CA + 1}], %[An]"), Op(f"s_mov_b64 s[{S_CB}:{S_CB + 1}], %[Bn]")]
+        if fp4:
+            last_pre += [Op(f"s_mov_b64 s[{S_CSA}:{S_CSA + 1}], %[mxan]"), Op(f"s_mov_b64 s[{S_CSB}:{S_CSB + 1}], %[mxbn]")]
+        P["last_pre"] = last_pre
+        P["last0"] = self.step(0, True, True)
+        P["last1"] = self.step(1, True, False)
         # the accumulators may be read by vector instructions 18 wait states after the last MFMA
-        e("s_nop 7")
-        e("s_nop 7")
-        e("s_nop 7")
+        end = [Op("s_nop 7"), Op("s_nop 7"), Op("s_nop 7")]
         if fp4:
             # the buffer that holds the next tile's first scale group
-            e(f"s_xor_b32 %[scbuf], s{S_SCN}, {SCBUF}")
+            end.append(Op(f"s_xor_b32 %[scbuf], s{S_SCN}, {SCBUF}"))
+        P["end"] = end
+        return P
+
+    # ---- text ---------------------------------------------------------------------------------------------
+    def wait_text(self, w):
+        """the instructions of one wait site: a single s_waitcnt, or a choice by the history flags"""
+        vals = w.vals
+        distinct = sorted(set(vals.values()))
+        if len(distinct) == 1:
+            return [f"s_waitcnt vmcnt({distinct[0]})"]
+        self.lbl += 1
+        L = lambda x: f"W4_W{self.lbl}{x}_%="
+        out = []
+        if set(vals) == {"s", "f"}:
+            out += [f"s_cmp_lg_u32 s{S_AFTER}, 0", f"s_cbranch_scc1 {L('f')}", f"s_waitcnt vmcnt({vals['s']})", f"s_branch {L('z')}",
+                    f"{L('f')}:", f"s_waitcnt vmcnt({vals['f']})", f"{L('z')}:"]
+            return out
+        order = [("a", "%[first]"), ("d", "%[fe]"), ("b", "%[nst]")]
+        for k, flag in order:
+            if k in vals:
+                out += [f"s_cmp_lg_u32 {flag}, 0", f"s_cbranch_scc1 {L(k)}"]
+        if "c" in vals:
+            out += [f"s_waitcnt vmcnt({vals['c']})", f"s_branch {L('z')}"]
+        for k, flag in order:
+            if k in vals:
+                out += [f"{L(k)}:", f"s_waitcnt vmcnt({vals[k]})", f"s_branch {L('z')}"]
+        out.append(f"{L('z')}:")
+        return out
+
+    def lines(self, ops):
+        out = []
+        for o in ops:
+            if isinstance(o, WaitVm):
+                ls = self.wait_text(o)
+            else:
+                ls = [o.text]
+            for s in ls:
+                if "nomfma" in self.lab and s.startswith("v_mfma"):
+                    continue
+                if "nodma" in self.lab and s.startswith("global_load_lds"):
+                    continue
+                if "noread" in self.lab and s.startswith("ds_read"):
+                    continue
+                if "nobar" in self.lab and s.startswith("s_barrier"):
+                    continue
+                if "novm" in self.lab and s.startswith("s_waitcnt vmcnt"):
+                    continue
+                if "nolgk" in self.lab and s.startswith("s_waitcnt lgkmcnt"):
+                    continue
+                out.append(s)
+        return out
+
+    def program(self):
+        P = self.parts()
+        T = lambda name: self.lines(P[name])
+        out = T("setup")
+        out += ["s_cmp_eq_u32 %[first], 0", "s_cbranch_scc1 W4_RESUME%="]
+        out += T("prologue") + ["s_branch W4_ENTRY%=", "W4_RESUME%=:"] + T("resume") + ["W4_ENTRY%=:"]
+        if self.scaled_epi:
+            # (22 fragment reads follow: a wait for "at most 15 outstanding" then covers these 16)
+            out += ["s_cmp_eq_u32 %[fe], 0", "s_cbranch_scc1 W4_NOSC%="] + T("entry_fe") + ["W4_NOSC%=:"]
+        out += T("entry")
+        out += ["s_cmp_lg_u32 %[fe], 0", "s_cbranch_scc1 W4_FE%="]
+        out += T("first0") + ["s_branch W4_FIRST1%=", "W4_FE%=:"] + T("first0_fe") + ["W4_FIRST1%=:"] + T("first1")
+        out += [f"s_sub_u32 s{S_CNT}, %[kh], 2", f"s_cmp_eq_u32 s{S_CNT}, 0", "s_cbranch_scc1 W4_LAST%=", "W4_LOOP%=:"]
+        out += T("steady0") + T("steady1")
+        out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_lg_u32 s{S_CNT}, 0", "s_cbranch_scc1 W4_LOOP%=", "W4_LAST%=:"]
+        out += T("last_pre") + T("last0") + T("last1") + T("end")
+        return out
 
     def text(self):
-        return "".join(f'  "{l}\\n\\t"\n' for l in self.out)
+        return "".join(f'  "{l}\\n\\t"\n' for l in self.program())
+
+    # ---- checker ----------------------------------------------------------------------------------------------
+    def check(self):
+        """Replays the vector-memory operations of every history a tile can have (first tile of the
+        workgroup; after a tile whose epilogue ran as compiled code with 32 stores, or with an unknown
+        number -- tried with none and with many; after a tile whose epilogue is fused into this one) for
+        tiles of 4, 6 and 8 K steps, two tiles in a row, and checks at every wait that the number it
+        allows in flight does not exceed the number of operations issued after the awaited group."""
+        P = self.parts()
+        worst = {}
+
+        def run(seq):
+            """seq: list of (part name, step number, history key or None)"""
+            q = []       # tags in issue order
+            for name, step, hist in seq:
+                if name == "cstores":
+                    q += [("CST", step)] * hist
+                    continue
+                for o in P[name]:
+                    if isinstance(o, WaitVm):
+                        grp = (o.awaits[0], o.awaits[1] + step)
+                        key = hist if hist in o.vals else ("s" if "s" in o.vals else None)
+                        assert key is not None, (name, step, hist, o.vals)
+                        n = o.vals[key]
+                        idx = max((i for i, t in enumerate(q) if t == grp), default=-1)
+                        assert idx >= 0 or grp[1] < -2 or True
+                        allowed = len(q) - 1 - idx
+                        assert n <= allowed, f"{self.kind}: {name} step {step} history {hist}: waits vmcnt({n}) for {grp}, only {allowed} younger operations exist"
+                        worst[(name, o.awaits, key)] = min(worst.get((name, o.awaits, key), 99), allowed - n)
+                    elif o.vm is not None:
+                        q.append((o.vm[0], o.vm[1] + step))
+            return q
+
+        def tile(base, ksteps, hist0, after_hist):
+            """parts of one tile whose step 0 is number `base`"""
+            s = [("first0_fe" if hist0 == "d" else "first0", base, hist0), ("first1", base + 1, hist0)]
+            h = "f"
+            for it in range(2, ksteps - 2, 2):
+                s += [("steady0", base + it, h), ("steady1", base + it + 1, "s")]
+                h = "s"
+            s += [("last0", base + ksteps - 2, h), ("last1", base + ksteps - 1, "s")]
+            return s
+
+        for k in (4, 6, 8):
+            for hist, nstores in (("b", NST), ("c", 0), ("c", 50), ("d", 0)):
+                seq = [("prologue", 0, "a")] + tile(0, k, "a", None)
+                seq += [("cstores", k, nstores)] + tile(k, k, hist, None)
+                seq += [("cstores", 2 * k, NST)] + tile(2 * k, k, "b", None)
+                run(seq)
+        return worst
 
 
-def clobbers():
-    names = [f"v{i}" for i in range(192)] + ["v240", "v241"] + [f"a{i}" for i in range(256)] + [f"s{i}" for i in range(70, 83)]
+def clobbers(kind):
+    """registers the statement writes that are not operands of it"""
+    v = list(range(192)) + [240, 241] if kind == "fp4" else list(range(160))
+    names = [f"v{i}" for i in v] + [f"a{i}" for i in range(256)] + [f"s{i}" for i in range(70, 90)]
     names += ["memory", "vcc", "scc", "m0"]
     lines = []
     for i in range(0, len(names), 16):
@@ -359,12 +562,15 @@ def clobbers():
 def main():
     what = sys.argv[1]
     if what == "clobbers":
-        sys.stdout.write(clobbers())
+        sys.stdout.write(clobbers(sys.argv[2]))
         return
-    import os
-    every = int(os.environ.get("W4GEN_DMA_EVERY", "1" if what == "fp8" else "2"))
-    g = Gen(what, every, [x for x in os.environ.get("W4GEN_LAB", "").split(",") if x])
-    g.kloop()
+    if what == "check":
+        for kind in ("fp8", "fp4", "bf16", "f16"):
+            w = Gen(kind).check()
+            print(kind, "ok; smallest slack per wait site:", min(w.values()), "largest:", max(w.values()))
+        return
+    g = Gen(what, [x for x in os.environ.get("W4GEN_LAB", "").split(",") if x])
+    g.check()
     sys.stdout.write(g.text())
 
 

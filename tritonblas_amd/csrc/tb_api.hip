@@ -77,7 +77,8 @@ struct Hooks {
   int panel = -1;               // TB_PANEL=<n>: column panel width of the tile order (-1: the library's)
   int no_column_split = 0, force_column_split = 0;
   int quant_div64 = 0;          // TB_QUANT_DIV64=1: the quantiser's kernel for 2^31 items and more at any size
-  int lab = 0;                  // TB_DEBUG=<bits>: only acted on by kernels built with TB_LAB_HOOKS
+  int lab = 0;                  // TB_DEBUG=<bits>: 4 = the 4-wave kernels store every tile with their compiled epilogue (none fused
+                                // into the next K loop); 1, 2 = only acted on by kernels built with TB_LAB_HOOKS
 };
 Hooks g_hooks;
 std::once_flag g_hooks_once;
@@ -141,7 +142,7 @@ const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, 
   const Variant* v; int n;
   variant_table(dt, &v, &n);
   // the hand-scheduled 4-wave kernels run K steps in pairs and have no Stream-K form
-  auto usable = [&](const Variant& x) { return !x.k_step_pairs || (!need_sk && k > 0 && k % (2 * (int64_t)x.bk) == 0); };
+  auto usable = [&](const Variant& x) { return !x.k_step_pairs || (!need_sk && k >= 4 * (int64_t)x.bk && k % (2 * (int64_t)x.bk) == 0); };
   const int want = hooks().waves;
   if (want && fast)
     for (int i = 0; i < n; ++i)
