@@ -77,6 +77,34 @@ def streamk_segments(pid, grid, total_tiles, sk_tiles, iters_per_tile):
     return out
 
 
+def streamk_walk_last_owner(wg, grid, total_tiles, sk_tiles, iters_per_tile):
+    """The order in which the LIBRARY's Stream-K kernel walks the same iteration range (the range is the
+    reference's, streamk_iter_range above; the walk is not: the reference's first segment owns the tile
+    and spins on locks of later programs, streamk_gemm.py:248-324, which needs every program resident).
+    Here `wg` is the raw workgroup id, the range is walked from its end, and the workgroup holding a
+    tile's last iterations finishes it.  Returns [(tile, k_first, k_last_exclusive, kind, waits_for)]
+    in processing order; kind is "publish" or "owner", waits_for the workgroup ids whose partials the
+    owner adds, in that order."""
+    start, last = streamk_iter_range(wg, grid, total_tiles, sk_tiles, iters_per_tile)
+    q, r = divmod(sk_tiles * iters_per_tile, grid)
+    out = []
+    while start < last:
+        tile = (last - 1) // iters_per_tile
+        tile_first = tile * iters_per_tile
+        begin = max(tile_first, start)
+        if last != tile_first + iters_per_tile:
+            out.append((tile, begin - tile_first, last - tile_first, "publish", []))
+        else:
+            waits, cur, nxt = [], begin, wg - 1
+            while cur > tile_first:
+                waits.append(nxt)
+                cur -= q + (1 if nxt < r else 0)
+                nxt -= 1
+            out.append((tile, begin - tile_first, last - tile_first, "owner", waits))
+        last = begin
+    return out
+
+
 def ws_slot_range(pid, total_tiles, num_xcds, counters_per_xcd):
     """Flat work-stealing queue a workgroup pulls from:
     include/tritonblas/kernels/persistent_gemm_work_stealing.py:296-314.

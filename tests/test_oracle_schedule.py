@@ -71,6 +71,45 @@ def test_streamk_covers_every_iteration_once(tiles, grid, ipt):
         assert pubs == list(range(owner + 1, owner + 1 + len(pubs)))
 
 
+@pytest.mark.parametrize("tiles,grid,ipt", [(64, 256, 112), (300, 256, 7), (5, 8, 3), (3, 7, 1), (10, 4, 5), (256, 256, 9),
+                                            (1, 256, 100), (2, 256, 5), (16, 200, 32)])
+def test_streamk_last_owner_walk_waits_only_for_started_workgroups(tiles, grid, ipt):
+    """The library's walk of the Stream-K range: every iteration once; a workgroup publishes at most one
+    partial and does so before anything else; the owner of a tile holds its last iteration and waits
+    exactly for the workgroups that hold the rest, all with lower ids (started earlier by the hardware),
+    each of which publishes that tile."""
+    sk_tiles = S.streamk_partition(tiles, grid)
+    if sk_tiles == 0:
+        sk_tiles = min(tiles, 1)       # (the host would take the whole-tile path; exercise the walk anyway)
+    full = tiles - sk_tiles
+    covered, publishes, owners = {}, {}, {}
+    for wg in range(grid):
+        walk = S.streamk_walk_last_owner(wg, grid, tiles, sk_tiles, ipt)
+        kinds = [w[3] for w in walk]
+        assert kinds.count("publish") <= 1 and (kinds.count("publish") == 0 or kinds[0] == "publish")
+        for tile, k0, k1, kind, waits in walk:
+            assert full <= tile < tiles and 0 <= k0 < k1 <= ipt
+            for k in range(k0, k1):
+                assert (tile, k) not in covered
+                covered[(tile, k)] = wg
+            if kind == "publish":
+                assert k1 < ipt
+                publishes[(tile, wg)] = (k0, k1)
+            else:
+                assert k1 == ipt
+                owners[tile] = (wg, k0, waits)
+    assert set(covered) == {(t, k) for t in range(full, tiles) for k in range(ipt)}
+    for tile, (wg, k0, waits) in owners.items():
+        assert all(w < wg for w in waits) and waits == list(range(wg - 1, wg - 1 - len(waits), -1))
+        need = k0
+        for w in waits:                      # nearest first: each partial ends where the previous began
+            a, b = publishes[(tile, w)]
+            assert b == need
+            need = a
+        assert need == 0
+    assert len(owners) == sk_tiles
+
+
 @pytest.mark.parametrize("tiles,xcds,cpx,grid", [(3584, 8, 1, 256), (1024, 8, 4, 256), (100, 8, 8, 256), (7, 8, 8, 256),
                                                  (513, 8, 4, 304), (64, 8, 8, 512)])
 def test_work_stealing_queues_partition_the_tiles(tiles, xcds, cpx, grid):

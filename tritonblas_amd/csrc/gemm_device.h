@@ -1105,7 +1105,7 @@ enum : int { WK_FULL = 0, WK_SK_PUBLISH = 1, WK_SK_OWNER = 2 };
 struct Work {
   TileCtx tc;
   int it0, it1, kind;
-  int64_t seg_end, tile_end;  // Stream-K owner: global iteration where its segment / its tile ends
+  int64_t seg_begin, tile_first;  // Stream-K owner: global iteration where its segment / its tile begins
 };
 
 __device__ __forceinline__ void plain_tile(const GemmParams& p, int tile, int BM, int BN, TileCtx& tc) {
@@ -1167,6 +1167,7 @@ __device__ __forceinline__ bool grouped_tile(const GemmParams& p, int phase, int
 template <class T, bool SK>
 struct Sched {
   int pid, G;
+  int sk_id;              // Stream-K: position of this workgroup's iteration range = its raw workgroup id
   int next_tile;          // static / Stream-K data-parallel phase
   int step;               // work stealing: queue visit index
   int64_t start, last, q, rem;  // Stream-K iteration range of this workgroup
@@ -1177,6 +1178,7 @@ struct Sched {
     G = gridDim.x;
     gphase = p.mode == MODE_GROUPED ? grouped_phase(p, G) : 0;
     pid = blockIdx.x;
+    sk_id = blockIdx.x;
     if (p.mode != MODE_WS && p.num_xcds > 1) pid = chiplet_transform_chunked(pid, G, p.num_xcds, p.chunk);
     next_tile = pid;
     step = 0;
@@ -1185,14 +1187,18 @@ struct Sched {
     if (p.mode == MODE_SK) {
       const int64_t total_sk = (int64_t)p.sk_tiles * p.k_iters;
       q = total_sk / G; rem = total_sk % G;
-      start = (int64_t)dp_tiles * p.k_iters + pid * q + min((int64_t)pid, rem);
-      last = (int64_t)dp_tiles * p.k_iters + (pid + 1) * q + min((int64_t)pid + 1, rem);
+      // The iteration ranges follow the order in which the hardware starts workgroups (the raw id, not
+      // the XCD-remapped one): a tile is finished by the workgroup that holds its LAST iterations, so
+      // every wait is for a workgroup with a lower id, which has been started already -- the exchange
+      // does not need the whole grid to be resident.
+      start = (int64_t)dp_tiles * p.k_iters + sk_id * q + min((int64_t)sk_id, rem);
+      last = (int64_t)dp_tiles * p.k_iters + (sk_id + 1) * q + min((int64_t)sk_id + 1, rem);
     }
     if (p.mode == MODE_WS && p.cu_mask && p.cu_mask[pid] == 0) step = 1 << 30;  // masked out: nothing to do
   }
 
   __device__ __forceinline__ bool next(const GemmParams& p, Work& w, int* s_bcast, int tid) {
-    w.it0 = 0; w.it1 = p.k_iters; w.kind = WK_FULL; w.seg_end = w.tile_end = 0;
+    w.it0 = 0; w.it1 = p.k_iters; w.kind = WK_FULL; w.seg_begin = w.tile_first = 0;
     if (p.mode == MODE_STATIC) {
       if (next_tile >= p.total_tiles) return false;
       plain_tile(p, next_tile, T::BM, T::BN, w.tc);
@@ -1294,18 +1300,21 @@ struct Sched {
       next_tile += G;
       return true;
     }
+    // The range is walked from its end: the piece that does not reach its tile's end (at most one,
+    // the head of the range's last tile) comes first and is published at once; the pieces that do
+    // reach a tile's end finish that tile, adding what lower workgroups published long before.
     if (start >= last) return false;
     const int ipt = p.k_iters;
-    const int tile = (int)(start / ipt);
+    const int tile = (int)((last - 1) / ipt);
     const int64_t tile_first = (int64_t)tile * ipt;
     const int64_t tile_end = tile_first + ipt;
-    const int64_t end = min(tile_end, last);
+    const int64_t begin = max(tile_first, start);
     plain_tile(p, tile, T::BM, T::BN, w.tc);
-    w.it0 = (int)(start - tile_first);
-    w.it1 = (int)(end - tile_first);
-    w.kind = (start != tile_first) ? WK_SK_PUBLISH : WK_SK_OWNER;
-    w.seg_end = end; w.tile_end = tile_end;
-    start = end;
+    w.it0 = (int)(begin - tile_first);
+    w.it1 = (int)(last - tile_first);
+    w.kind = (last != tile_end) ? WK_SK_PUBLISH : WK_SK_OWNER;
+    w.seg_begin = begin; w.tile_first = tile_first;
+    last = begin;
     return true;
   }
 };
@@ -1342,22 +1351,23 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
       continue;
     }
     if (w.kind == WK_SK_PUBLISH) {
-      // not the tile's first segment: publish the partial, tagged with this launch's epoch
-      partial_store<T>(p.P + (size_t)sched.pid * (T::BM * T::BN), acc, li.tid);
+      // not the tile's last segment: publish the partial, tagged with this launch's epoch
+      partial_store<T>(p.P + (size_t)sched.sk_id * (T::BM * T::BN), acc, li.tid);
       __builtin_amdgcn_s_waitcnt(0x0070);   // this wave's write-through stores have left the CU
       __syncthreads();                      // ... and so have everybody else's
       if (li.tid == 0) {
         // one L2 write-back for the workgroup (it covers every wave's stores), then the flag
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        __hip_atomic_store(p.flags + sched.pid, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.flags + sched.sk_id, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       continue;
     }
     if (w.kind == WK_SK_OWNER) {
-      // owner of the tile: add the partials of the following workgroups in ascending order
-      int nxt = sched.pid + 1;
-      int64_t cur_end = w.seg_end;
-      while (cur_end < w.tile_end) {
+      // owner of the tile (it holds the last iterations): add the partials of the workgroups before it,
+      // nearest first -- a fixed order, so the sum is the same in every launch
+      int nxt = sched.sk_id - 1;
+      int64_t cur_begin = w.seg_begin;
+      while (cur_begin > w.tile_first) {
         if (li.tid == 0) {
           uint32_t spins = 0;
           int ok = 1;
@@ -1371,7 +1381,8 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
         int ok = s_bcast;
         __syncthreads();
         if (!ok) {
-          // a partner never published (it is not resident, or the bound is too tight): the tile cannot
+          // a partner did not publish within the bound (the bound is too tight, or the device is shared
+          // with something that starves it): the tile cannot
           // be finished.  It is stored as NaN so that nobody mistakes stale memory for a result, and the
           // status word tells the host.
           failed = true;
@@ -1383,8 +1394,8 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
           break;
         }
         partial_add<T>(p.P + (size_t)nxt * (T::BM * T::BN), acc, li.tid);
-        cur_end += sched.q + (nxt < sched.rem ? 1 : 0);
-        ++nxt;
+        cur_begin -= sched.q + (nxt < sched.rem ? 1 : 0);
+        --nxt;
       }
     }
     }

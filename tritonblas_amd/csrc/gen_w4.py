@@ -309,8 +309,20 @@ class Gen:
         pre[xs] += self.frag_read(self.vA(4), 0, p, 4)
         xops = ops_b + lo + sc
         span = 5 * nm - 2 - xs
+        m0_slots = set()
+
+        def place(slot, op):
+            """A copy needs one wait state between the write of m0 and its use: the MFMA of the slot is
+            that instruction (m0 setup in front of it, the copy right behind)."""
+            if len(op) == 3 and "nodma" not in self.lab and "m0nop" not in self.lab:
+                assert slot not in m0_slots
+                m0_slots.add(slot)
+                pre[slot].append(op[0])
+                post[slot].insert(0, op[2])
+            else:
+                post[slot] += op
         for n, op in enumerate(xops):
-            post[xs + n * span // len(xops)] += op
+            place(xs + n * span // len(xops), op)
         post[5 * nm - 2] += adv_b
         pre[2 * nm] += self.frag_read(self.vA(5), 0, p, 5)
         pre[3 * nm] += self.frag_read(self.vA(6), 0, p, 6)
@@ -348,7 +360,7 @@ class Gen:
             post[a1] += self.frag_read(self.vA(1), 0, q, 1)
             post[a2] += self.frag_read(self.vA(2), 0, q, 2)
         for n, op in enumerate(hi):
-            post[tail0 + n * (tail - 2) // len(hi)] += op
+            place(tail0 + n * (tail - 2) // len(hi), op)
         post[total - 2] += adv_a
         for m in range(total):
             out += pre[m]

@@ -401,9 +401,11 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     plan->ws_need = WS_FLAGS_OFF;
   } else if (j.schedule == TB_SCHED_STREAMK) {
     p.mode = MODE_SK;
-    // (a requested grid that cannot be co-resident for the kernel that really runs -- the caller sized it
-    // for another tile, e.g. the operands turned out to need the gather kernel -- gives way to the
-    // library's own choice: owners wait for later workgroups, so all of them must be on the device)
+    // (a requested grid larger than what is resident at once for the kernel that really runs -- the caller
+    // sized it for another tile, e.g. the operands turned out to need the gather kernel -- gives way to
+    // the library's own choice.  Correctness does not need residency: a tile's owner only waits for
+    // workgroups with lower ids, which the hardware has started before it.  But an owner that waits
+    // occupies its CU, so a grid beyond residency only adds waiting.)
     int64_t g = j.grid;
     if (g <= 0 || g > resident) {
       tb_problem pr;
@@ -419,7 +421,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     }
     const bool whole_only = g == total;   // exactly one workgroup per tile (however many fit at once): nothing to share
     if (whole_only) g = std::min<int64_t>(total, resident);
-    if (g > resident) return TB_ERR_BAD_SCHEDULE;  // owners spin on later workgroups: all must be resident
+    if (g > resident) return TB_ERR_BAD_SCHEDULE;
     grid = (int)g;
     p.sk_tiles = whole_only ? 0 : (int32_t)(total % grid);
     if (p.sk_tiles == 0) {
