@@ -10,7 +10,9 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtritonblas_amd.so")
+# TRITONBLAS_AMD_LIB names another build of the library (measurement builds of the kernels: see the
+# W4GEN_LAB options of csrc/gen_w4.py); the default is the in-tree one
+LIB_PATH = os.environ.get("TRITONBLAS_AMD_LIB") or os.path.join(_HERE, "lib", "libtritonblas_amd.so")
 
 # ---- enums (mirrors of the header) -------------------------------------------------------------
 TB_OK = 0

@@ -100,8 +100,9 @@ class Gen:
         # how far (in MFMAs) into row blocks 1 and 5 the two sync points of a K step sit
         self.xoff = int(os.environ.get("W4GEN_XOFF", str(self.nm // 2)))
         self.yoff = int(os.environ.get("W4GEN_YOFF", str(self.nm // 2)))
-        # measurement builds (W4GEN_LAB=nomfma,nodma,noread,nobar,novm,nolgk): leave one kind of
-        # instruction out to time the rest; results are then meaningless
+        # measurement builds (W4GEN_LAB=nomfma,nodma,dmaonce,noread,nobar,novm,nolgk,m0nop): leave one kind of
+        # instruction out to time the rest; results are then meaningless.  dmaonce = nodma except for the
+        # first tile's entry copies, so that the LDS holds real operand data for the MFMAs to chew on.
         self.lab = set(lab)
         self.v_coff = 238 if self.fp4 else 240
         self.v_lane4, self.v_sa_rd, self.v_sb_rd = 241, 242, 243
@@ -314,7 +315,7 @@ class Gen:
         def place(slot, op):
             """A copy needs one wait state between the write of m0 and its use: the MFMA of the slot is
             that instruction (m0 setup in front of it, the copy right behind)."""
-            if len(op) == 3 and "nodma" not in self.lab and "m0nop" not in self.lab:
+            if len(op) == 3 and not ({"nodma", "dmaonce", "m0nop"} & self.lab):
                 assert slot not in m0_slots
                 m0_slots.add(slot)
                 pre[slot].append(op[0])
@@ -465,7 +466,7 @@ class Gen:
         out.append(f"{L('z')}:")
         return out
 
-    def lines(self, ops):
+    def lines(self, ops, keep_dma=False):
         out = []
         for o in ops:
             if isinstance(o, WaitVm):
@@ -475,7 +476,7 @@ class Gen:
             for s in ls:
                 if "nomfma" in self.lab and s.startswith("v_mfma"):
                     continue
-                if "nodma" in self.lab and s.startswith("global_load_lds"):
+                if ("nodma" in self.lab or ("dmaonce" in self.lab and not keep_dma)) and s.startswith("global_load_lds"):
                     continue
                 if "noread" in self.lab and s.startswith("ds_read"):
                     continue
@@ -493,7 +494,7 @@ class Gen:
         T = lambda name: self.lines(P[name])
         out = T("setup")
         out += ["s_cmp_eq_u32 %[first], 0", "s_cbranch_scc1 W4_RESUME%="]
-        out += T("prologue") + ["s_branch W4_ENTRY%=", "W4_RESUME%=:"] + T("resume") + ["W4_ENTRY%=:"]
+        out += self.lines(P["prologue"], keep_dma=True) + ["s_branch W4_ENTRY%=", "W4_RESUME%=:"] + T("resume") + ["W4_ENTRY%=:"]
         if self.scaled_epi:
             # (22 fragment reads follow: a wait for "at most 15 outstanding" then covers these 16)
             out += ["s_cmp_eq_u32 %[fe], 0", "s_cbranch_scc1 W4_NOSC%="] + T("entry_fe") + ["W4_NOSC%=:"]
