@@ -3,6 +3,7 @@ benchmarks/tritonblas_matmul.py; shape lists of datasets/generate_grid*.py."""
 import csv
 
 import pytest
+import torch
 import yaml
 
 REFERENCE_COLUMNS = ["m", "n", "k", "mnk", "macro_tile", "bytes", "flops", "tritonblas_gflops", "a_type", "b_type", "c_type",
@@ -70,6 +71,37 @@ def test_cu_sweep_steps():
     assert cu_sweep_steps(256, 8, 32, 100)[-1] == 8                                    # at least one CU per XCD stays
     assert _fieldnames([{"active_cus": 8, "m": 1}]) == ["active_cus"] + REFERENCE_COLUMNS
     assert _fieldnames([{"m": 1}]) == REFERENCE_COLUMNS and _fieldnames([]) == REFERENCE_COLUMNS
+
+
+def test_masked_cu_sweep_parent(tmp_path, monkeypatch):
+    """--cu-sweep --cu-mask (reference benchmarks/tritonblas_matmul.py:381-412): the parent asks a child for the CU
+    counts, then runs one child per step with the balanced ROC_GLOBAL_CU_MASK of that step and without the sweep /
+    output flags, and concatenates their JSON rows.  The children are faked here; the parent must not touch a GPU."""
+    import json
+    from types import SimpleNamespace
+    from tritonblas_amd.benchmarks import matmul_bench
+    from tritonblas_amd.benchmarks.common import build_balanced_hex_mask
+    calls = []
+
+    def fake_child(argv_tail, env=None):
+        calls.append((list(argv_tail), None if env is None else env.get("ROC_GLOBAL_CU_MASK")))
+        if "--_cu-info" in argv_tail:
+            return SimpleNamespace(returncode=0, stdout="[256, 8, 32]\n", stderr="")
+        active = int(argv_tail[argv_tail.index("--_active-cus") + 1])
+        return SimpleNamespace(returncode=0, stdout="noise\n" + json.dumps([{"active_cus": active, "m": 1}]) + "\n", stderr="")
+
+    monkeypatch.setattr(matmul_bench, "_child", fake_child)
+    monkeypatch.setattr(torch.cuda, "current_device", lambda: (_ for _ in ()).throw(AssertionError("GPU call in the parent")))
+    dst = tmp_path / "out.csv"
+    matmul_bench.main(["--input-yaml", "shapes.yaml", "--output-csv", str(dst), "--work-stealing", "--cu-sweep", "--cu-mask",
+                       "--cu-sweep-max-remove", "2", "--n-repeat", "3"])
+    assert calls[0][0] == ["--input-yaml", "shapes.yaml", "--_cu-info"]
+    assert [c[1] for c in calls[1:]] == [None, build_balanced_hex_mask(1, 8, 32), build_balanced_hex_mask(2, 8, 32)]
+    for argv_tail, _ in calls[1:]:
+        assert argv_tail[:5] == ["--input-yaml", "shapes.yaml", "--work-stealing", "--n-repeat", "3"]
+        assert "--cu-sweep" not in argv_tail and "--cu-mask" not in argv_tail and "--output-csv" not in argv_tail
+    rows = list(csv.DictReader(dst.open()))
+    assert [int(r["active_cus"]) for r in rows] == [256, 248, 240]
 
 
 @pytest.mark.gpu

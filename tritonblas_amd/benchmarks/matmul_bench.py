@@ -3,7 +3,7 @@
     python -m tritonblas_amd.benchmarks.matmul_bench --input-yaml shapes.yaml --output-csv out.csv
         [--enable-streamk | --work-stealing] [--checkcorrectness] [--init_type randn|hpl|trig_float|zeros]
         [--shuffle-bench] [--csv-write-freq N] [--n-warmup W] [--n-repeat R]
-        [--global-atomic | --hierarchical] [--counters-per-xcd C] [--cu-sweep [--cu-sweep-max-remove R]]
+        [--global-atomic | --hierarchical] [--counters-per-xcd C] [--cu-sweep [--cu-mask] [--cu-sweep-max-remove R]]
 
 Input: a YAML list of {m, n, k, in_dtype, out_dtype, transA, transB} (in_dtype "fp4" selects the MXFP4
 GEMM).  Output: one CSV row per case with the column set of the reference's driver
@@ -13,13 +13,18 @@ Timing is the reference's do_bench loop (cache flush and workspace reset outside
 (benchmarks/tritonblas_matmul.py:78-111).
 --cu-sweep repeats the shape list with 0, 1, 2, ... CUs per XCD taken away (benchmarks/tritonblas_matmul.py:381-412):
 the selector is built with total_cus = active_cus = what is left, which sizes the launch grid, and with
---work-stealing the per-workgroup mask; rows gain a leading active_cus column.  The sweep runs in this process;
-to also fence the hardware, set the runtime's CU mask yourself (benchmarks.common.build_balanced_hex_mask
-gives the balanced mask strings the reference uses).
+--work-stealing the per-workgroup mask; rows gain a leading active_cus column.  That sweep runs in this process.
+--cu-sweep --cu-mask fences the hardware instead, as the reference does: every step runs in a child process with
+ROC_GLOBAL_CU_MASK set to the balanced mask of that step (benchmarks.common.build_balanced_hex_mask) and the library
+sized for the whole device; the parent starts its children before it makes any GPU call of its own (it asks a first
+child for the CU counts) and collects their rows as JSON.
 """
 import argparse
 import csv
+import json
+import os
 import random
+import subprocess
 import sys
 
 import torch
@@ -152,6 +157,50 @@ def cu_sweep_steps(full_cus, num_xcds, cus_per_xcd, max_remove):
     return [full_cus - r * num_xcds for r in range(min(max_remove, cus_per_xcd - 1) + 1)]
 
 
+def _child(argv_tail, env=None):
+    return subprocess.run([sys.executable, "-m", "tritonblas_amd.benchmarks.matmul_bench"] + argv_tail,
+                          capture_output=True, text=True, env=env)
+
+
+def masked_cu_sweep(args, argv):
+    """Balanced CU-mask sweep (reference benchmarks/tritonblas_matmul.py:381-412): step r runs the shape list
+    in a child process with the first r CUs of every XCD masked off by the runtime."""
+    from .common import build_balanced_hex_mask
+    info = _child(["--input-yaml", args.input_yaml, "--_cu-info"])
+    if info.returncode != 0:
+        raise RuntimeError("could not query the device: " + info.stderr[-500:])
+    full_cus, num_xcds, cus_per_xcd = json.loads(info.stdout.strip().splitlines()[-1])
+    # the child's arguments: everything but the sweep flags and the output file
+    tail, skip = [], False
+    for a in argv:
+        if skip:
+            skip = False
+        elif a in ("--cu-sweep", "--cu-mask"):
+            pass
+        elif a in ("--output-csv", "--cu-sweep-max-remove"):
+            skip = True
+        elif a.startswith("--output-csv=") or a.startswith("--cu-sweep-max-remove="):
+            pass
+        else:
+            tail.append(a)
+    rows = []
+    for r in range(min(args.cu_sweep_max_remove, cus_per_xcd - 1) + 1):
+        active = full_cus - r * num_xcds
+        env = os.environ.copy()
+        mask = build_balanced_hex_mask(r, num_xcds, cus_per_xcd)
+        if mask:
+            env["ROC_GLOBAL_CU_MASK"] = mask
+        else:
+            env.pop("ROC_GLOBAL_CU_MASK", None)
+        proc = _child(tail + ["--_active-cus", str(active)], env)
+        print(f"[active_cus={active}] {proc.stderr[-300:]}", file=sys.stderr, flush=True)
+        if proc.returncode != 0:
+            print(f"[active_cus={active}] child failed with status {proc.returncode}", file=sys.stderr)
+            continue
+        rows += json.loads(proc.stdout.strip().splitlines()[-1])
+    return rows
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--input-yaml", required=True)
@@ -166,7 +215,12 @@ def main(argv=None):
     ap.add_argument("--n-warmup", type=int, default=20)
     ap.add_argument("--n-repeat", type=int, default=100)
     ap.add_argument("--cu-sweep", action="store_true", help="repeat the shape list with CUs taken away from every XCD")
+    ap.add_argument("--cu-mask", action="store_true", help="with --cu-sweep: fence the hardware (ROC_GLOBAL_CU_MASK, one child "
+                                                           "process per step) instead of sizing the launch")
     ap.add_argument("--cu-sweep-max-remove", type=int, default=34, help="most CUs to take from one XCD")
+    # children of a --cu-mask sweep: print the CU counts / run the shape list and print the rows as JSON
+    ap.add_argument("--_cu-info", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--_active-cus", type=int, default=None, help=argparse.SUPPRESS)
     ap.add_argument("--counters-per-xcd", type=int, default=None, help="work-stealing queues per XCD (default: the selector's)")
     ap.add_argument("--global-atomic", action="store_true", help="work stealing from one device-wide counter")
     ap.add_argument("--hierarchical", action="store_true", help="work stealing from XCD-local queues, then a shared pool")
@@ -175,10 +229,34 @@ def main(argv=None):
         ap.error("--enable-streamk and --work-stealing select different schedules; give one")
     if args.global_atomic and args.hierarchical:
         ap.error("--global-atomic and --hierarchical are different queue layouts; give one")
+    if args.cu_mask and not args.cu_sweep:
+        ap.error("--cu-mask is a mode of --cu-sweep")
+    if args._cu_info:
+        from .common import get_cu_info
+        print(json.dumps(list(get_cu_info(torch.cuda.current_device()))))
+        return
+    if args.cu_sweep and args.cu_mask:
+        # (no GPU call in this process: the children own the device, one at a time)
+        res = masked_cu_sweep(args, argv if argv is not None else sys.argv[1:])
+        if args.output_csv:
+            write_csv(args.output_csv, res)
+        else:
+            w = csv.DictWriter(sys.stdout, fieldnames=_fieldnames(res))
+            w.writeheader()
+            w.writerows(res)
+        return
     common = dict(init_type=args.init_type, print_verbose=args.print_verbose, shuffle_benchmark=args.shuffle_bench,
                   write_csv_freq=args.csv_write_freq, enable_streamk=args.enable_streamk, work_stealing=args.work_stealing,
                   check_correctness=args.checkcorrectness, n_warmup=args.n_warmup, n_repeat=args.n_repeat,
                   counters_per_xcd=args.counters_per_xcd, global_atomic=args.global_atomic, hierarchical=args.hierarchical)
+    if args._active_cus is not None:
+        # child of a masked sweep: the runtime fences the CUs, the library is sized for the whole device
+        # (reference benchmarks/tritonblas_matmul.py:421: active_cus = total_cus under a CU mask)
+        real_stdout, sys.stdout = sys.stdout, sys.stderr
+        res = bench_matmul(args.input_yaml, output_csv=None, **common)
+        sys.stdout = real_stdout
+        print(json.dumps([{"active_cus": args._active_cus, **r} for r in res]))
+        return
     if args.cu_sweep:
         from .common import get_cu_info
         res = []
