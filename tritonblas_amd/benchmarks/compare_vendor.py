@@ -1,0 +1,112 @@
+"""Side-by-side timing of this library and the vendor library PyTorch dispatches to (hipBLASLt through
+torch.matmul / torch._scaled_mm) on the same tensors.
+
+    python -m tritonblas_amd.benchmarks.compare_vendor [--shapes fp8,bf16] [--steps 40] [--settle-ms 40]
+
+Cases: "fp8" = a8w8 8192x28672x8192 with per-row / per-column scales (torch._scaled_mm row-wise is the
+same operation; its tensor-wise form, one scale per tensor, is the simpler problem the vendor ships a
+hand-written kernel for) and "bf16" = 8192^3 with K-major operands.  Every timing starts after
+`settle-ms` of untimed launches of the same call (the engine clock needs tens of milliseconds of load
+to settle) and is the average of `steps` back-to-back launches between two events.  One JSON line per
+case on stdout.  Run it under `rocprofv3 --kernel-trace --stats` or `--pmc` to see the kernels behind
+each call.
+"""
+import argparse
+import json
+import sys
+import time
+
+import torch
+
+
+def timed(fn, steps, settle_ms):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def case_fp8(steps, settle_ms, dev):
+    import tritonblas_amd as tb
+    import tritonblas_amd.utils as U
+    m, n, k = 8192, 28672, 8192
+    g = torch.Generator(device=dev).manual_seed(2)
+    a = torch.randn(m, k, device=dev, generator=g).bfloat16()
+    w = torch.randn(n, k, device=dev, generator=g).bfloat16()
+    aq, sa = U.quantize_tensor_per_channel(a, torch.float8_e4m3fn, axis=1)
+    wq, sw = U.quantize_tensor_per_channel(w, torch.float8_e4m3fn, axis=1)
+    del a, w
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    sel = tb.OrigamiMatmulSelector(m, n, k, aq.dtype, wq.dtype, c.dtype, dev)
+    out = {"case": "fp8 a8w8 8192x28672x8192, bf16 out", "flops": 2.0 * m * n * k}
+    out["this_library_ms"] = timed(lambda: tb.matmul_a8w8_lt(aq, wq.T, sa, sw, c, sel, None), steps, settle_ms)
+    sa2, sw2 = sa.reshape(m, 1).contiguous(), sw.reshape(1, n).contiguous()
+    try:
+        ref = torch._scaled_mm(aq, wq.T, scale_a=sa2, scale_b=sw2, out_dtype=torch.bfloat16)
+        out["vendor_rowwise_ms"] = timed(lambda: torch._scaled_mm(aq, wq.T, scale_a=sa2, scale_b=sw2, out_dtype=torch.bfloat16, out=c),
+                                         steps, settle_ms)
+        tb.matmul_a8w8_lt(aq, wq.T, sa, sw, c, sel, None)
+        torch.cuda.synchronize()
+        rows = slice(0, 512)
+        out["rel_fro_between_the_two"] = float(((c[rows].float() - ref[rows].float()).norm() / ref[rows].float().norm()).item())
+        del ref
+    except Exception as e:   # (the row-wise form is not available in every PyTorch build)
+        out["vendor_rowwise_error"] = str(e)[:200]
+    one_a, one_w = torch.ones((), device=dev), torch.ones((), device=dev)
+    try:
+        out["vendor_tensorwise_ms"] = timed(lambda: torch._scaled_mm(aq, wq.T, scale_a=one_a, scale_b=one_w, out_dtype=torch.bfloat16, out=c),
+                                            steps, settle_ms)
+    except Exception as e:
+        out["vendor_tensorwise_error"] = str(e)[:200]
+    return out
+
+
+def case_bf16(steps, settle_ms, dev):
+    import tritonblas_amd as tb
+    m = n = k = 8192
+    g = torch.Generator(device=dev).manual_seed(3)
+    a = (torch.rand(m, k, device=dev, generator=g) * 2 - 1).bfloat16()
+    b = (torch.rand(n, k, device=dev, generator=g) * 2 - 1).bfloat16().T
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, c.dtype, dev)
+    out = {"case": "bf16 8192x8192x8192, K-major operands", "flops": 2.0 * m * n * k}
+    out["this_library_ms"] = timed(lambda: tb.matmul_lt(a, b, c, sel, None), steps, settle_ms)
+    out["vendor_ms"] = timed(lambda: torch.matmul(a, b, out=c), steps, settle_ms)
+    return out
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--shapes", default="fp8,bf16")
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--settle-ms", type=float, default=40.0)
+    args = ap.parse_args(argv)
+    dev = torch.device("cuda", torch.cuda.current_device())
+    for name in args.shapes.split(","):
+        fn = {"fp8": case_fp8, "bf16": case_bf16}.get(name.strip())
+        if fn is None:
+            print(f"unknown case {name!r}", file=sys.stderr)
+            return 2
+        r = fn(args.steps, args.settle_ms, dev)
+        for key in list(r):
+            if key.endswith("_ms"):
+                r[key.replace("_ms", "_tflops")] = round(r["flops"] / r[key] / 1e9, 1)
+                r[key] = round(r[key], 4)
+        print(json.dumps(r), flush=True)
+        torch.cuda.empty_cache()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

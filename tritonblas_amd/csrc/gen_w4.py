@@ -101,7 +101,7 @@ class Gen:
         self.xoff = int(os.environ.get("W4GEN_XOFF", str(self.nm // 2)))
         self.yoff = int(os.environ.get("W4GEN_YOFF", str(self.nm // 2)))
         # measurement builds (W4GEN_LAB=nomfma,nodma,dmaonce,noread,nobar,novm,nolgk,m0nop): leave one kind of
-        # instruction out to time the rest; results are then meaningless.  dmaonce = nodma except for the
+        # instruction out (noscale: the MXFP4 kernel's scale copies and scale reads) to time the rest; results are then meaningless.  dmaonce = nodma except for the
         # first tile's entry copies, so that the LDS holds real operand data for the MFMAs to chew on.
         self.lab = set(lab)
         self.v_coff = 238 if self.fp4 else 240
@@ -485,6 +485,10 @@ class Gen:
                 if "novm" in self.lab and s.startswith("s_waitcnt vmcnt"):
                     continue
                 if "nolgk" in self.lab and s.startswith("s_waitcnt lgkmcnt"):
+                    continue
+                if ({"noscale", "noscaleread"} & self.lab) and s.startswith("ds_read_u16"):
+                    continue
+                if ({"noscale", "noscaledma"} & self.lab) and s.startswith("global_load_lds_dwordx4 v23") and s[27] in "4567":
                     continue
                 out.append(s)
         return out
