@@ -18,7 +18,7 @@ def _load():
     return mod
 
 
-@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "f16"])
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "f16", "i8"])
 def test_wait_counts_hold_for_every_history(kind):
     gen = _load()
     slack = gen.Gen(kind).check()
@@ -39,7 +39,7 @@ def test_checker_catches_a_wait_that_is_too_loose():
         g.check()
 
 
-@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16"])
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "i8"])
 def test_program_shape(kind):
     """one MFMA per accumulator tile and K slice in every step; the fused epilogue stores 32 times"""
     gen = _load()

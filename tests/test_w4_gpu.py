@@ -161,8 +161,13 @@ def _launcher(kind, m, n, k, seed):
     """returns (run, want): run() launches the 256x256 tile kernel the hooks select and returns C on the host"""
     import tritonblas_amd as tb
     from tritonblas_amd.matmul import persistent_matmul_lt
-    if kind == "fp8":
-        aq, bq, sa, sb = _fp8_case(m, n, k, seed)
+    if kind in ("fp8", "i8"):
+        if kind == "fp8":
+            aq, bq, sa, sb = _fp8_case(m, n, k, seed)
+        else:
+            g = torch.Generator().manual_seed(seed)
+            aq, sa = OG.quantize_per_channel_int8(torch.randn(m, k, generator=g), axis=1)
+            bq, sb = OG.quantize_per_channel_int8(torch.randn(k, n, generator=g), axis=0)
         a, b, sad, sbd = aq.cuda(), bq.T.contiguous().cuda().T, sa.cuda(), sb.cuda()
 
         def run():
@@ -171,6 +176,8 @@ def _launcher(kind, m, n, k, seed):
             c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
             persistent_matmul_lt(a, b, c, sel, None, a_scale=sad, b_scale=sbd, quantized=True)
             return c.cpu()
+        if kind == "i8":
+            return run, OG.ref_gemm_int8(aq, bq, torch.bfloat16, a_scale=sa, b_scale=sb).to(torch.bfloat16)
         return run, OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
     if kind == "fp4":
         xq, wq, xs, ws = _fp4_case(m, n, k, seed)
@@ -196,7 +203,7 @@ def _launcher(kind, m, n, k, seed):
     return run, OG.ref_gemm(a_cpu, bt_cpu.T, torch.float32).to(torch.bfloat16)
 
 
-@pytest.mark.parametrize("kind,bk", [("fp8", 128), ("fp4", 256), ("bf16", 64)])
+@pytest.mark.parametrize("kind,bk", [("fp8", 128), ("fp4", 256), ("bf16", 64), ("i8", 128)])
 @pytest.mark.parametrize("m,n,steps,grid", [(512, 768, 4, 1), (512, 768, 6, 2), (300, 500, 8, 1), (1280, 768, 10, 3), (1100, 1300, 4, 2),
                                             (4096, 8192, 4, 0)])
 def test_fused_epilogue(kind, bk, m, n, steps, grid, tb_option):
@@ -217,7 +224,7 @@ def test_fused_epilogue(kind, bk, m, n, steps, grid, tb_option):
     tb_option("lab", 0)
     fused = run()
     again = run()
-    assert OG.rel_fro_error(fused.float(), want.float()) <= (1e-3 if kind == "bf16" else TOL_Q)
+    assert OG.rel_fro_error(fused.float(), want.float()) <= (1e-3 if kind in ("bf16", "i8") else TOL_Q)
     assert torch.equal(compiled.view(torch.int16), eight.view(torch.int16))
     assert torch.equal(fused.view(torch.int16), compiled.view(torch.int16))
     assert torch.equal(again.view(torch.int16), fused.view(torch.int16))

@@ -5,6 +5,7 @@
 namespace tb {
 
 const Variant g_variants_i8[] = {
+    make_variant_w4<W4Tile<DT_I8>>(),
     make_variant<Tile<DT_I8, 256, 256, 128, 2, 4, LAY_K, LAY_K, 1, true, 2>>(),
     make_variant<Tile<DT_I8, 128, 128, 128, 2, 2, LAY_K, LAY_K, 2, true, 2>>(),
     make_variant<Tile<DT_I8, 64, 64, 128, 2, 2, LAY_K, LAY_K, 4, true, 2>>(),

@@ -1,4 +1,4 @@
-// The hand-scheduled 4-wave 256x256 kernels (FP8, MXFP4, bf16, fp16), see gemm_w4.h.
+// The hand-scheduled 4-wave 256x256 kernels (FP8, MXFP4, bf16, fp16, int8), see gemm_w4.h.
 #include "gemm_w4.h"
 
 namespace tb {
@@ -8,6 +8,7 @@ const void* w4_kernel(int dt) {
   if (dt == DT_FP4) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP4>>;
   if (dt == DT_BF16) return (const void*)&gemm_kernel_w4<W4Tile<DT_BF16>>;
   if (dt == DT_F16) return (const void*)&gemm_kernel_w4<W4Tile<DT_F16>>;
+  if (dt == DT_I8) return (const void*)&gemm_kernel_w4<W4Tile<DT_I8>>;
   return nullptr;
 }
 

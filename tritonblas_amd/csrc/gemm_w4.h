@@ -47,12 +47,19 @@ __device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
   return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
-// accumulator register a[N] (written by the K loop statement; the compiler never allocates these)
-template <int N>
+// accumulator register a[N] (written by the K loop statement; the compiler never allocates these);
+// INT: the K loop left an int32 sum there
+template <int N, bool INT = false>
 __device__ __forceinline__ float acc_read() {
-  float x;
-  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
-  return x;
+  if constexpr (INT) {
+    int x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
+    return (float)x;
+  } else {
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N));
+    return x;
+  }
 }
 
 // what the K loop needs to know about one output tile
@@ -126,7 +133,7 @@ __device__ __forceinline__ void epilogue_w4(const GemmParams& p, const TileCtx& 
       float v[8];
       static_for<8>([&](auto E) {
         constexpr int e = decltype(E)::value;
-        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3))>();
+        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3)), T::DT == DT_I8>();
       });
       const int m = tc.m0 + ln.wm0 + i * 16 + ln.r;
       if (m >= tc.m_lim || nvalid <= 0) return;
@@ -198,7 +205,7 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
       float v[8];
       static_for<8>([&](auto E) {
         constexpr int e = decltype(E)::value;
-        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3))>();
+        v[e] = acc_read<((i * 8 + 2 * q + (e >> 2)) * 4 + (e & 3)), T::DT == DT_I8>();
       });
       if (p.sa) {
 #pragma unroll
@@ -215,8 +222,11 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
 #ifdef W4_LAB_NOSTORE
       if (p.debug == 12345)         // measurement build: no stores (the condition keeps the code alive)
 #endif
-      if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off offset:%2 nt" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
-      else asm volatile("global_store_dwordx4 %0, %1, off offset:%2" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
+      // (the s_nop: a store of more than 8 bytes reads its data registers a little after it issues, and the
+      // compiler, which inserts the wait states for its own stores, cannot see into this statement -- without
+      // them the int8 kernel's next conversion overwrote the first data register for some lanes)
+      if constexpr (NT) asm volatile("global_store_dwordx4 %0, %1, off offset:%2 nt\n\ts_nop 1" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
+      else asm volatile("global_store_dwordx4 %0, %1, off offset:%2\n\ts_nop 1" : : "v"(dst), "v"(pk), "n"(q * 64) : "memory");
     });
   });
 }
@@ -230,7 +240,7 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
-  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16, "element types with a generated K loop");
+  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16 || T::DT == DT_I8, "element types with a generated K loop");
   // two stages, the FP4 scale buffers (16 KB), 1 KB per wave for epilogue scales, the schedule's broadcast word
   __shared__ __attribute__((aligned(16))) uint8_t lds[W4_LDS_BYTES];
   int& s_bcast = *(int*)(lds + W4_LDS_BYTES - 16);
@@ -290,7 +300,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   int fe = 0;                       // 1: the previous tile's sums are still in the accumulators
   const uint8_t* cprev = (const uint8_t*)p.C;   // C[first row of the wave's quarter][its first column] of that tile
   const bool fe_shape = p.c_line && !p.bias && p.c_type == DT_BF16 && p.c_sm < (1 << 26) && (p.debug & 4) == 0 &&
-                        ((T::DT == DT_FP8) == (p.sa != nullptr));
+                        ((T::DT == DT_FP8 || T::DT == DT_I8) == (p.sa != nullptr));
   // a lane's C offset from cprev, the same in every row block (rows of a row block are c_sm apart);
   // lane * 4; where the lane finds the scales of its rows 16 i + r and of its columns 32 q + 8 g + 0..7
   v4i eo;
@@ -309,22 +319,32 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     w4_tile_args<T>(p, wnext.tc, ln, nxt);
     const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
                       (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
-    const bool regs = T::DT == DT_FP8 && fast && p.sa;    // the K loop copies this tile's scale vectors
+    const bool regs = (T::DT == DT_FP8 || T::DT == DT_I8) && fast && p.sa;    // the K loop copies this tile's scale vectors
     const uint8_t *sA = uniform(cur.A), *sB = uniform(cur.B), *sAn = uniform(nxt.A), *sBn = uniform(nxt.B);
     const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst), s_fe = uniform(fe);
     const uint8_t* s_cprev = uniform(cprev);
     scbuf = uniform(scbuf);
-    if constexpr (T::DT == DT_FP8) {
+    if constexpr (T::DT == DT_FP8 || T::DT == DT_I8) {
       // (a tile without scales or off the fast path loads 512 bytes of its operands instead; nobody uses them)
       const uint8_t* s_sap = uniform(regs ? (const uint8_t*)(p.sa + w.tc.m0 + ln.wm0) : cur.A);
       const uint8_t* s_sbp = uniform(regs ? (const uint8_t*)(w.tc.sb + w.tc.n0 + ln.wn0) : cur.B);
-      asm volatile(
+      if constexpr (T::DT == DT_FP8) {
+        asm volatile(
 #include "w4_kloop_fp8.inc"
-          : [scbuf] "+s"(scbuf)
-          : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
-          :
+            : [scbuf] "+s"(scbuf)
+            : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
+            :
 #include "w4_clobbers_fp8.inc"
-      );
+        );
+      } else {
+        asm volatile(
+#include "w4_kloop_i8.inc"
+            : [scbuf] "+s"(scbuf)
+            : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
+            :
+#include "w4_clobbers_i8.inc"
+        );
+      }
     } else if constexpr (T::DT == DT_BF16) {
       asm volatile(
 #include "w4_kloop_bf16.inc"

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Writes the hand-scheduled K loop of the 4-wave 256x256 tile kernels (gemm_w4.h) as inline-assembly text.
 
-    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: fp4, bf16, f16)
+    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: fp4, bf16, f16, i8)
     python3 gen_w4.py clobbers fp8 > w4_clobbers_fp8.inc
     python3 gen_w4.py check                          (walks every kind through the wait-count checker)
 
@@ -91,9 +91,10 @@ class WaitVm:
 
 class Gen:
     def __init__(self, kind, lab=()):
-        self.kind = kind                # "fp8" | "fp4" | "bf16" | "f16"
+        self.kind = kind                # "fp8" | "fp4" | "bf16" | "f16" | "i8"
         self.fp4 = kind == "fp4"        # (the only kind with E8M0 scale operands)
-        self.scaled_epi = kind == "fp8"  # the fused epilogue multiplies by sa[m] * sb[n]
+        self.scaled_epi = kind in ("fp8", "i8")  # the fused epilogue multiplies by sa[m] * sb[n]
+        self.int_acc = kind == "i8"      # int32 sums: converted to fp32 where they leave the accumulators
         self.nm = 8 if kind == "fp8" else 16      # MFMAs per row block (FP8: one of K = 128 per fragment pair; others: two half-K ones)
         self.nsc = 4 if self.scaled_epi else 0    # copies of the tile's own epilogue scales (step 1)
         self.lbl = 0
@@ -187,6 +188,8 @@ class Gen:
         c = "0" if (zero and ks == 0) else f"a[{acc}:{acc + 3}]"
         if self.kind in ("bf16", "f16"):
             return Op(f"v_mfma_f32_16x16x32_{self.kind} a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}")
+        if self.kind == "i8":
+            return Op(f"v_mfma_i32_16x16x64_i8 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}")
         return Op(f"v_mfma_scale_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}, "
                   f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
 
@@ -203,6 +206,9 @@ class Gen:
                 base = (i * 8 + 2 * q + h) * 4
                 for x in range(4):
                     out.append(Op(f"v_accvgpr_read_b32 v{e[x]}, a{base + x}"))
+                if self.int_acc:
+                    for x in range(4):
+                        out.append(Op(f"v_cvt_f32_i32 v{e[x]}, v{e[x]}"))
                 if self.scaled_epi:
                     for x in range(4):
                         out.append(Op(f"v_mul_f32 v{s}, v{self.v_sa + i}, v{self.v_sb + q * 8 + h * 4 + x}"))
@@ -582,7 +588,7 @@ def main():
         sys.stdout.write(clobbers(sys.argv[2]))
         return
     if what == "check":
-        for kind in ("fp8", "fp4", "bf16", "f16"):
+        for kind in ("fp8", "fp4", "bf16", "f16", "i8"):
             w = Gen(kind).check()
             print(kind, "ok; smallest slack per wait site:", min(w.values()), "largest:", max(w.values()))
         return

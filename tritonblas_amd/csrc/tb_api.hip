@@ -285,7 +285,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (j.num_groups > 0) at_once = 0;
     // (the 4-wave kernels have no Stream-K form and no 8-bit output path)
     v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw,
-                     (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) || j.c_type == TB_FP8_E4M3, j.K);
+                     (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) || j.c_type == TB_FP8_E4M3 || j.c_type == TB_I8, j.K);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
@@ -425,8 +425,16 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     grid = (int)g;
     p.sk_tiles = whole_only ? 0 : (int32_t)(total % grid);
     if (p.sk_tiles == 0) {
-      // nothing to share: the same tiles on the whole-tile kernel (identical results, no workspace)
+      // nothing to share: the same tiles on the whole-tile kernel (identical results, no workspace) --
+      // which may be the hand-scheduled 4-wave form of this tile, ruled out above only for its lack of
+      // a Stream-K tail (same tile, one workgroup per CU either way, bit-identical sums)
       p.mode = MODE_STATIC;
+      if (v->fast && j.c_type != TB_FP8_E4M3 && j.c_type != TB_I8) {
+        const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K);
+        if (w && w->k_step_pairs && w->bm == v->bm && w->bn == v->bn && w->bk == v->bk &&
+            std::max(1, std::min(w->minb, hw.lds_bytes / w->lds_bytes)) == occ)
+          v = w;
+      }
     } else {
       plan->ws_flags_off = WS_FLAGS_OFF;
       plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
