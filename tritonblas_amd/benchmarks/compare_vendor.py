@@ -1,13 +1,15 @@
 """Side-by-side timing of this library and the vendor library PyTorch dispatches to (hipBLASLt through
 torch.matmul / torch._scaled_mm) on the same tensors.
 
-    python -m tritonblas_amd.benchmarks.compare_vendor [--shapes fp8,bf16] [--steps 40] [--settle-ms 40]
+    python -m tritonblas_amd.benchmarks.compare_vendor [--shapes fp8,bf16,decode] [--steps 40] [--settle-ms 40]
 
 Cases: "fp8" = a8w8 8192x28672x8192 with per-row / per-column scales (torch._scaled_mm row-wise is the
 same operation; its tensor-wise form, one scale per tensor, is the simpler problem the vendor ships a
 hand-written kernel for) and "bf16" = 8192^3 with K-major operands.  Every timing starts after
 `settle-ms` of untimed launches of the same call (the engine clock needs tens of milliseconds of load
-to settle) and is the average of `steps` back-to-back launches between two events.  One JSON line per
+to settle) and is the average of `steps` back-to-back launches between two events.  "decode" = a8w8
+32x8192x28672 (the 235 MB weight is the traffic): timed back to back and with the caches flushed before
+every launch (do_bench), next to a plain device copy of as many bytes under the same flush.  One JSON line per
 case on stdout.  Run it under `rocprofv3 --kernel-trace --stats` or `--pmc` to see the kernels behind
 each call.
 """
@@ -86,6 +88,37 @@ def case_bf16(steps, settle_ms, dev):
     return out
 
 
+def case_decode(steps, settle_ms, dev):
+    import tritonblas_amd as tb
+    import tritonblas_amd.utils as U
+    m, n, k = 32, 8192, 28672
+    g = torch.Generator(device=dev).manual_seed(22)
+    a = torch.randn(m, k, device=dev, generator=g).bfloat16()
+    w = torch.randn(n, k, device=dev, generator=g).bfloat16()
+    aq, sa = U.quantize_tensor_per_channel(a, torch.float8_e4m3fn, axis=1)
+    wq, sw = U.quantize_tensor_per_channel(w, torch.float8_e4m3fn, axis=1)
+    del a, w
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    sel = tb.OrigamiMatmulSelector(m, n, k, aq.dtype, wq.dtype, c.dtype, dev, streamk=True)
+    cfg = tb.matmul_preamble(sel, dev)
+    ours = lambda: tb.matmul_a8w8_lt(aq, wq.T, sa, sw, c, sel, cfg, enable_streamk=True)
+    sa2, sw2 = sa.reshape(m, 1).contiguous(), sw.reshape(1, n).contiguous()
+    vendor = lambda: torch._scaled_mm(aq, wq.T, scale_a=sa2, scale_b=sw2, out_dtype=torch.bfloat16, out=c)
+    nbytes = m * k + n * k + m * n * 2 + (m + n) * 4
+    out = {"case": "fp8 a8w8 decode 32x8192x28672, bf16 out", "flops": 2.0 * m * n * k, "bytes": nbytes}
+    out["this_library_ms"] = timed(ours, steps * 4, settle_ms / 4)
+    out["this_library_flushed_ms"] = tb.do_bench(ours, n_warmup=5, n_repeat=40, return_mode="median")
+    try:
+        out["vendor_rowwise_ms"] = timed(vendor, steps * 4, settle_ms / 4)
+        out["vendor_rowwise_flushed_ms"] = tb.do_bench(vendor, n_warmup=5, n_repeat=40, return_mode="median")
+    except Exception as e:
+        out["vendor_rowwise_error"] = str(e)[:200]
+    x = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    y = torch.empty_like(x)
+    out["plain_copy_of_as_many_bytes_flushed_ms"] = tb.do_bench(lambda: y.copy_(x), n_warmup=3, n_repeat=20, return_mode="median")
+    return out
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="fp8,bf16")
@@ -94,14 +127,17 @@ def main(argv=None):
     args = ap.parse_args(argv)
     dev = torch.device("cuda", torch.cuda.current_device())
     for name in args.shapes.split(","):
-        fn = {"fp8": case_fp8, "bf16": case_bf16}.get(name.strip())
+        fn = {"fp8": case_fp8, "bf16": case_bf16, "decode": case_decode}.get(name.strip())
         if fn is None:
             print(f"unknown case {name!r}", file=sys.stderr)
             return 2
         r = fn(args.steps, args.settle_ms, dev)
         for key in list(r):
             if key.endswith("_ms"):
-                r[key.replace("_ms", "_tflops")] = round(r["flops"] / r[key] / 1e9, 1)
+                if "bytes" in r:
+                    r[key.replace("_ms", "_TBps")] = round(r["bytes"] / r[key] / 1e9, 2)
+                else:
+                    r[key.replace("_ms", "_tflops")] = round(r["flops"] / r[key] / 1e9, 1)
                 r[key] = round(r[key], 4)
         print(json.dumps(r), flush=True)
         torch.cuda.empty_cache()
