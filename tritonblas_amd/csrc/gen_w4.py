@@ -544,7 +544,7 @@ class Gen:
                         assert key is not None, (name, step, hist, o.vals)
                         n = o.vals[key]
                         idx = max((i for i, t in enumerate(q) if t == grp), default=-1)
-                        assert idx >= 0 or grp[1] < -2 or True
+                        assert idx >= 0, f"{self.kind}: {name} step {step} waits for {grp}, which nobody issued"
                         allowed = len(q) - 1 - idx
                         assert n <= allowed, f"{self.kind}: {name} step {step} history {hist}: waits vmcnt({n}) for {grp}, only {allowed} younger operations exist"
                         worst[(name, o.awaits, key)] = min(worst.get((name, o.awaits, key), 99), allowed - n)
