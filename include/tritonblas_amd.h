@@ -143,7 +143,11 @@ typedef struct tb_gemm_desc {
                                  the workspace is refused with TB_ERR_BAD_ARGUMENT), and never a value an
                                  earlier launch on this workspace used since it was last zeroed: count
                                  upwards (flags are not cleared between launches, a stale flag of an equal
-                                 epoch would pass for published)                                          */
+                                 epoch would pass for published).  TB_EPOCH_ON_DEVICE instead of a number
+                                 lets the workspace count for itself (control word 2, advanced by the last
+                                 workgroup of every such launch): the form to use when launches are replayed
+                                 from a captured graph, whose arguments cannot change.  Do not mix the two
+                                 forms on one workspace without zeroing it in between                      */
   uint32_t spin_limit;        /* Stream-K: bound on flag polls per wait; 0 = default                 */
   /* work stealing only (config.py:23, persistent_gemm_work_stealing.py:70-81): */
   const int32_t* cu_mask;     /* device int32[cu_mask_len] or NULL; workgroup i leaves at once when
@@ -172,17 +176,19 @@ size_t tb_workspace_bytes(const tb_gemm_desc* desc);
 /* tb_gemm without a workspace from the caller and without any allocation: the queue counters, Stream-K
  * flags and partial tiles live in a buffer of TB_STATIC_WORKSPACE_BYTES that is part of the library's
  * device image (every GPU the library runs on holds it until the process ends).  desc->workspace,
- * workspace_bytes and epoch are ignored (the library keeps its own epoch per device); a launch that
+ * workspace_bytes and epoch are ignored (the buffer counts its own launches, TB_EPOCH_ON_DEVICE); a launch that
  * needs more than TB_STATIC_WORKSPACE_BYTES is refused with TB_ERR_WORKSPACE.  No counterpart in the
  * reference: it is for callers that cannot allocate device memory where they launch -- code under HIP
  * graph capture, tight serving loops, harnesses that forbid it.  All calls on one GPU share the buffer:
  * calls that may overlap in time (different streams) race; calls on one stream do not. */
 #define TB_STATIC_WORKSPACE_BYTES (16u << 20)
+#define TB_EPOCH_ON_DEVICE 0xFFFFFFFFu
 int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream);
 
 /* Byte offsets of the regions of a workspace: [0, 256) control words -- word 0 is the status (set to 1
  * when a Stream-K wait ran into spin_limit: the tile concerned was then stored as NaN; cleared only by the
- * caller), word 1 counts finished work-stealing workgroups; *counters_offset: work-stealing queue
+ * caller), word 1 counts workgroups that have finished (work stealing, and Stream-K with
+ * TB_EPOCH_ON_DEVICE), word 2 is the workspace's own launch count for TB_EPOCH_ON_DEVICE; *counters_offset: work-stealing queue
  * counters, one per 256-byte line; *flags_offset: Stream-K flags (one word per workgroup), the partial
  * tiles follow at the next 256-byte boundary behind `grid` flags.  Replaces the separate buffers of
  * matmul_preamble (config.py:86-134). */

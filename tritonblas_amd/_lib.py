@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("TRITONBLAS_AMD_LIB") or os.path.join(_HERE, "lib", "l
 
 # ---- enums (mirrors of the header) -------------------------------------------------------------
 TB_OK = 0
+TB_EPOCH_ON_DEVICE = 0xFFFFFFFF   # tb_gemm_desc.epoch: the workspace counts its own Stream-K launches
 TB_ERR_NULL_POINTER, TB_ERR_BAD_SHAPE, TB_ERR_BAD_DTYPE, TB_ERR_BAD_LAYOUT, TB_ERR_BAD_TILE = -1, -2, -3, -4, -5
 TB_ERR_WORKSPACE, TB_ERR_BAD_SCHEDULE, TB_ERR_LAUNCH, TB_ERR_NO_DEVICE, TB_ERR_BAD_ARGUMENT = -6, -7, -8, -9, -10
 TB_F16, TB_BF16, TB_FP8_E4M3, TB_FP4_E2M1, TB_F32, TB_I8 = 0, 1, 2, 3, 4, 5

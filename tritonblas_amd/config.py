@@ -63,7 +63,9 @@ class MatmulConfig:
         return self.workspace
 
     def next_epoch(self) -> int:
-        """Epochs only count upwards; before they would wrap the workspace is cleared."""
+        """A host-side epoch for callers that drive tb_gemm themselves with this config's workspace (the
+        package's own launches let the workspace count: _lib.TB_EPOCH_ON_DEVICE; do not mix the two on one
+        workspace without reset()).  Epochs only count upwards; before they would wrap the workspace is cleared."""
         if self.epoch >= 0x7FFFFFFF:
             self.workspace.zero_()
             self.epoch = 0

@@ -24,7 +24,8 @@ enum : int { WS_QUEUES = 0, WS_GLOBAL = 1, WS_HIERARCHICAL = 2 };   // how work-
 enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
 
 // Word offsets inside the control block at the head of a workspace.
-enum : int { CTL_STATUS = 0, CTL_DONE = 1, CTL_WORDS = 64 };
+enum : int { CTL_STATUS = 0, CTL_DONE = 1, CTL_EPOCH = 2, CTL_WORDS = 64 };
+constexpr uint32_t EPOCH_ON_DEVICE = 0xFFFFFFFFu;   // GemmParams::epoch: the workspace's own count tags the launch
 constexpr int COUNTER_STRIDE = 64;  // ints between queue counters: one 256-byte line each
 
 // Measurement hooks of the K loop (skip the copies or the MFMAs; results are then meaningless) exist
@@ -1340,6 +1341,13 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   sched.init(p);
   Work w;
   bool failed = false;
+  // The tag of this launch's partial tiles: the caller's epoch, or one more than the count the
+  // workspace keeps itself (control word CTL_EPOCH, which the last workgroup to leave advances) --
+  // the form a launch replayed from a captured graph needs, whose arguments cannot change.
+  uint32_t epoch = p.epoch;
+  if constexpr (SK) {
+    if (p.epoch == EPOCH_ON_DEVICE) epoch = __hip_atomic_load(p.ctl + CTL_EPOCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  }
   while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
     __syncthreads();  // the previous item's store staging may still be read by slower waves
     mainloop<T, !SK>(p, w.tc, w.it0, w.it1, acc, lds, li);
@@ -1358,7 +1366,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
       if (li.tid == 0) {
         // one L2 write-back for the workgroup (it covers every wave's stores), then the flag
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        __hip_atomic_store(p.flags + sched.sk_id, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.flags + sched.sk_id, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       continue;
     }
@@ -1371,7 +1379,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
         if (li.tid == 0) {
           uint32_t spins = 0;
           int ok = 1;
-          while (__hip_atomic_load(p.flags + nxt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != p.epoch) {
+          while (__hip_atomic_load(p.flags + nxt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != epoch) {
             if (++spins >= p.spin_limit) { ok = 0; break; }
             __builtin_amdgcn_s_sleep(2);
           }
@@ -1403,6 +1411,14 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   }
   if constexpr (SK) {
     if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
+    if (p.epoch == EPOCH_ON_DEVICE && p.mode == MODE_SK && li.tid == 0) {
+      // every workgroup has read the count before it gets here, so the last one to leave may advance it
+      const uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
+      if (done == gridDim.x - 1) {
+        __hip_atomic_store(p.ctl + CTL_EPOCH, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
   }
   if (!SK && p.mode == MODE_WS && li.tid == 0) {
     // the last workgroup to leave rearms the queues for the next launch

@@ -651,11 +651,9 @@ static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 struct ScratchState {
   void* ptr = nullptr;
   int status = TB_ERR_NO_DEVICE;
-  uint32_t epoch = 0;
 };
 ScratchState g_scratch[MAX_DEVICES];
 std::once_flag g_scratch_once[MAX_DEVICES];
-std::mutex g_scratch_mu;
 
 void init_scratch(int dev) {
   void* ptr = nullptr;
@@ -663,11 +661,6 @@ void init_scratch(int dev) {
   if (e != hipSuccess || !ptr) { (void)hipGetLastError(); g_scratch[dev].status = TB_ERR_NO_DEVICE; return; }
   g_scratch[dev].ptr = ptr;
   g_scratch[dev].status = TB_OK;
-}
-
-// clears words [0, n) of a buffer (used instead of a memset node, which a caller's graph capture must not record)
-__global__ void fill_zero_kernel(uint32_t* ptr, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) ptr[i] = 0u;
 }
 
 int job_from_gemm(const tb_gemm_desc* d, Job* j) {
@@ -828,17 +821,10 @@ int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream) {
   if (sc.status != TB_OK) return sc.status;
   j.workspace = sc.ptr;
   j.workspace_bytes = SCRATCH_BYTES;   // (a launch that needs more is refused with TB_ERR_WORKSPACE)
-  {
-    // the array keeps the last call's contents: Stream-K flags are told apart by a per-device epoch that
-    // only counts upwards; when it would wrap, the flags are cleared first (the queue counters rearm themselves)
-    std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (sc.epoch == 0xFFFFFFFFu) {
-      hipLaunchKernelGGL(fill_zero_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, (uint32_t*)sc.ptr, SCRATCH_BYTES / 4);
-      if (hipGetLastError() != hipSuccess) return TB_ERR_LAUNCH;
-      sc.epoch = 0;
-    }
-    j.epoch = ++sc.epoch;
-  }
+  // The array keeps the last call's contents (it starts as zeros): the queue counters rearm themselves, and
+  // Stream-K launches are told apart by the count the workspace keeps in its own control block -- so the
+  // call records nothing that a replay of a captured graph would repeat wrongly.
+  j.epoch = TB_EPOCH_ON_DEVICE;
   return launch_columns(j, (hipStream_t)stream);
 }
 

@@ -147,7 +147,9 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
                 config = _stream_config(dev)
             ws = config.ensure(need)
             d.workspace, d.workspace_bytes = C.c_void_p(ws.data_ptr()), ws.numel()
-            d.epoch = config.next_epoch()
+            # (the workspace tags Stream-K launches with its own count: nothing in the descriptor changes from
+            # call to call, so a launch captured in a graph can be replayed)
+            d.epoch = _lib.TB_EPOCH_ON_DEVICE
             d.spin_limit = int(getattr(config, "spin_limit", 0) or 0)
     with _on_device(dev):
         _lib.check(lib.tb_gemm(d, _lib.stream_handle(dev)), "tb_gemm")
