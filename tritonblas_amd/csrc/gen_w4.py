@@ -101,7 +101,7 @@ class Gen:
         # how far (in MFMAs) into row blocks 1 and 5 the two sync points of a K step sit
         self.xoff = int(os.environ.get("W4GEN_XOFF", str(self.nm // 2)))
         self.yoff = int(os.environ.get("W4GEN_YOFF", str(self.nm // 2)))
-        # measurement builds (W4GEN_LAB=nomfma,nodma,dmaonce,noread,nobar,novm,nolgk,m0nop): leave one kind of
+        # measurement builds (W4GEN_LAB=nomfma,nodma,dmaonce,noread,nobar,novm,nolgk,m0nop,nostore): leave one kind of
         # instruction out (noscale: the MXFP4 kernel's scale copies and scale reads) to time the rest; results are then meaningless.  dmaonce = nodma except for the
         # first tile's entry copies, so that the LDS holds real operand data for the MFMAs to chew on.
         self.lab = set(lab)
@@ -491,6 +491,8 @@ class Gen:
                 if "novm" in self.lab and s.startswith("s_waitcnt vmcnt"):
                     continue
                 if "nolgk" in self.lab and s.startswith("s_waitcnt lgkmcnt"):
+                    continue
+                if "nostore" in self.lab and s.startswith("global_store"):
                     continue
                 if ({"noscale", "noscaleread"} & self.lab) and s.startswith("ds_read_u16"):
                     continue
