@@ -42,10 +42,12 @@ enum {
   TB_FP8_E4M3 = 2,  /* OCP e4m3fn                                                  */
   TB_FP4_E2M1 = 3,  /* two codes per byte, low nibble = even k (utils.py:585-587) */
   TB_F32 = 4,       /* operands (full fp32 products, 16x16x4 MFMA), output, bias, quantiser input */
-  TB_I8 = 5         /* operands (int32 sums, persistent_gemm.py:75); as output only with TB_I8 operands: fp32 epilogue
+  TB_I8 = 5,        /* operands (int32 sums, persistent_gemm.py:75); as output only with TB_I8 operands: fp32 epilogue
                        result truncated toward zero and saturated to [-128, 127]                    */
+  TB_FP8_E5M2 = 6   /* OCP e5m2, operands of tb_gemm only (the type utils.py:46 lists next to e4m3); both
+                       operands must have the same 8-bit format                                     */
 };
-/* TB_FP8_E4M3 is also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 operands: the fp32 epilogue
+/* TB_FP8_E4M3 is also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 or TB_FP8_E5M2 operands: the fp32 epilogue
  * result is clamped to +-448 and rounded to nearest even (the reference's a8w8 oracle,
  * tests/test_matmul_a8w8_lt.py:11-38). */
 

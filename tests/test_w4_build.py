@@ -20,8 +20,8 @@ HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
 def test_compiled_code_leaves_the_accumulators_alone(tmp_path):
     # (the generated K loops must exist: the library's build writes them)
-    subprocess.run(["make", "-C", CSRC, "-s"] + [f"w4_kloop_{k}.inc" for k in ("fp8", "fp4", "bf16", "f16", "i8")] +
-                   [f"w4_clobbers_{k}.inc" for k in ("fp8", "fp4", "bf16", "f16", "i8")], check=True)
+    subprocess.run(["make", "-C", CSRC, "-s"] + [f"w4_kloop_{k}.inc" for k in ("fp8", "e5m2", "fp4", "bf16", "f16", "i8")] +
+                   [f"w4_clobbers_{k}.inc" for k in ("fp8", "e5m2", "fp4", "bf16", "f16", "i8")], check=True)
     out = tmp_path / "w4.s"
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-Wno-unused-command-line-argument", "-Wno-pass-failed", "-Wno-inline-asm", "-S", "--cuda-device-only",
@@ -29,7 +29,7 @@ def test_compiled_code_leaves_the_accumulators_alone(tmp_path):
     subprocess.run(cmd, check=True, cwd=CSRC, stderr=subprocess.DEVNULL)
     text = out.read_text()
     kernels = re.findall(r"^(_ZN2tb14gemm_kernel_w4\S+):", text, re.M)
-    assert len(kernels) == 5
+    assert len(kernels) == 6
     assert "v_accvgpr_write" not in text and "v_accvgpr_mov" not in text
     # every accumulator read is one of ours: inside the generated loops (plain register names) or an
     # acc_read<N>() statement of the compiled epilogues (bracketed index)

@@ -18,7 +18,7 @@ def _load():
     return mod
 
 
-@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "f16", "i8"])
+@pytest.mark.parametrize("kind", ["fp8", "e5m2", "fp4", "bf16", "f16", "i8"])
 def test_wait_counts_hold_for_every_history(kind):
     gen = _load()
     slack = gen.Gen(kind).check()
@@ -39,13 +39,13 @@ def test_checker_catches_a_wait_that_is_too_loose():
         g.check()
 
 
-@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16", "i8"])
+@pytest.mark.parametrize("kind", ["fp8", "e5m2", "fp4", "bf16", "i8"])
 def test_program_shape(kind):
     """one MFMA per accumulator tile and K slice in every step; the fused epilogue stores 32 times"""
     gen = _load()
     g = gen.Gen(kind)
     parts = g.parts()
-    per_step = 64 if kind == "fp8" else 128
+    per_step = 64 if kind in ("fp8", "e5m2") else 128
     for name in ("first0", "first0_fe", "first1", "steady0", "steady1", "last0", "last1"):
         assert sum(1 for o in parts[name] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")) == per_step, name
     stores = [o for o in parts["first0_fe"] if not isinstance(o, gen.WaitVm) and o.text.startswith("global_store")]
@@ -56,3 +56,14 @@ def test_program_shape(kind):
     assert sum(1 for t in first if t.count("a[") == 1) == 64          # (no accumulator among the sources)
     steady = [o.text for o in parts["steady0"] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")]
     assert all(t.count("a[") == 2 for t in steady)
+
+
+def test_e5m2_differs_from_e4m3_only_in_the_format_field():
+    gen = _load()
+    a, b = gen.Gen("fp8").program(), gen.Gen("e5m2").program()
+    assert len(a) == len(b)
+    for x, y in zip(a, b):
+        if x.startswith("v_mfma"):
+            assert y == x + " cbsz:1 blgp:1"
+        else:
+            assert x == y

@@ -19,7 +19,7 @@ TB_OK = 0
 TB_EPOCH_ON_DEVICE = 0xFFFFFFFF   # tb_gemm_desc.epoch: the workspace counts its own Stream-K launches
 TB_ERR_NULL_POINTER, TB_ERR_BAD_SHAPE, TB_ERR_BAD_DTYPE, TB_ERR_BAD_LAYOUT, TB_ERR_BAD_TILE = -1, -2, -3, -4, -5
 TB_ERR_WORKSPACE, TB_ERR_BAD_SCHEDULE, TB_ERR_LAUNCH, TB_ERR_NO_DEVICE, TB_ERR_BAD_ARGUMENT = -6, -7, -8, -9, -10
-TB_F16, TB_BF16, TB_FP8_E4M3, TB_FP4_E2M1, TB_F32, TB_I8 = 0, 1, 2, 3, 4, 5
+TB_F16, TB_BF16, TB_FP8_E4M3, TB_FP4_E2M1, TB_F32, TB_I8, TB_FP8_E5M2 = 0, 1, 2, 3, 4, 5, 6
 TB_SCHED_PERSISTENT, TB_SCHED_WORK_STEALING, TB_SCHED_STREAMK = 0, 1, 2
 TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
 
@@ -157,7 +157,7 @@ def check(status: int, what: str = "tritonblas_amd"):
     raise RuntimeError(f"{what}: {msg} (status {status})")
 
 
-_DTYPES = {torch.float16: TB_F16, torch.bfloat16: TB_BF16, torch.float32: TB_F32, torch.float8_e4m3fn: TB_FP8_E4M3,
+_DTYPES = {torch.float16: TB_F16, torch.bfloat16: TB_BF16, torch.float32: TB_F32, torch.float8_e4m3fn: TB_FP8_E4M3, torch.float8_e5m2: TB_FP8_E5M2,
            torch.int8: TB_I8}
 
 

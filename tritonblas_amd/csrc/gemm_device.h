@@ -18,7 +18,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
-enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4, DT_I8 = 5 };
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4, DT_I8 = 5, DT_E5M2 = 6 };
+// the two 8-bit float formats (OCP e4m3 = DT_FP8, e5m2) share everything but the MFMA's format field
+constexpr bool is_f8(int dt) { return dt == DT_FP8 || dt == DT_E5M2; }
 enum : int { MODE_STATIC = 0, MODE_WS = 1, MODE_SK = 2, MODE_GROUPED = 3 };
 enum : int { WS_QUEUES = 0, WS_GLOBAL = 1, WS_HIERARCHICAL = 2 };   // how work-stealing workgroups find tiles
 enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
@@ -115,7 +117,7 @@ struct Tile {
   static constexpr int UPS = CPR * UPC;                                // units per K step
   static constexpr int EPU = (DT == DT_FP4) ? 2 : 1;                   // elements per unit
   static constexpr int BK = UPS * EPU;                                 // elements per K step
-  static constexpr int KS = (DT == DT_FP8) ? 8 : 4;                    // chunks one MFMA consumes per row
+  static constexpr int KS = is_f8(DT) ? 8 : 4;                         // chunks one MFMA consumes per row
   static constexpr int KSUB = CPR / KS;                                // MFMA k-slices per K step
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 16, TN = WTN / 16;
@@ -405,12 +407,12 @@ struct Operand {
 // ------------------------------------------------------------------------------------------------
 template <class T>
 struct Frag {
-  using type = typename std::conditional<T::DT == DT_FP8, v8i, v4i>::type;
+  using type = typename std::conditional<is_f8(T::DT), v8i, v4i>::type;
 
   // row: tile row of this lane (wave row base + 16*t + lane%16); g = lane/16; m = swizzle mask of row.
   __device__ static __forceinline__ type read(const uint8_t* lds, int row, int ks, int g, int m) {
     const uint8_t* rp = lds + row * T::BKB;
-    if constexpr (T::DT == DT_FP8) {
+    if constexpr (is_f8(T::DT)) {
       int c0 = ks * 8 + 2 * g;
       v4i lo = *(const v4i*)(rp + ((c0 ^ m) << 4));
       v4i hi = *(const v4i*)(rp + (((c0 + 1) ^ m) << 4));
@@ -444,8 +446,9 @@ __device__ __forceinline__ v4f mma(typename Frag<T>::type x, typename Frag<T>::t
   } else if constexpr (T::DT == DT_I8) {
     // exact int32 sums: the accumulator registers hold integers until the K loop ends
     return __builtin_bit_cast(v4f, __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, __builtin_bit_cast(v4i, c), 0, 0, 0));
-  } else if constexpr (T::DT == DT_FP8) {
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
+  } else if constexpr (is_f8(T::DT)) {
+    constexpr int FMT = T::DT == DT_E5M2 ? 1 : 0;   // format field of both operands: 0 = e4m3, 1 = e5m2
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, FMT, FMT, 0, 0, 0, 0);
   } else {
     v8i x8 = {x.x, x.y, x.z, x.w, 0, 0, 0, 0};
     v8i y8 = {y.x, y.y, y.z, y.w, 0, 0, 0, 0};
@@ -544,7 +547,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
       }
       // pin the issue order for the machine scheduler: B fragments and the first A fragment, then
       // alternately the next A fragment's reads and one row block of MFMAs
-      constexpr int RPF = (T::DT == DT_FP8) ? 2 : 1;  // LDS reads per fragment
+      constexpr int RPF = is_f8(T::DT) ? 2 : 1;  // LDS reads per fragment
       __builtin_amdgcn_sched_group_barrier(0x100, RPF * (T::TN + 1), 0);
 #pragma unroll
       for (int i = 0; i + 1 < T::TM; ++i) {
@@ -647,7 +650,7 @@ __device__ __forceinline__ void mainloop(const GemmParams& p, const TileCtx& tc,
     frag_t afn;
     auto request_b = [&](const uint8_t* sB, int ks, int j) { bf[j] = Frag<T>::read(sB, li.wn0 + j * 16 + li.r, ks, li.g, swm); };
     auto request_a = [&](const uint8_t* sA, int ks, int i) { return Frag<T>::read(sA, li.wm0 + i * 16 + li.r, ks, li.g, swm); };
-    constexpr int RPF = (T::DT == DT_FP8) ? 2 : 1;  // LDS reads per fragment
+    constexpr int RPF = is_f8(T::DT) ? 2 : 1;  // LDS reads per fragment
 
     // one block: slice KSV of the K step in stage (sA, sB).  `boundary` runs before the last row block;
     // afterwards the fragments of slice nks of stage (nA, nB) are requested.  After the last step of
@@ -1033,7 +1036,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc,
   if constexpr (T::DT == DT_I8) {
     if (p.c_type == DT_I8) { epilogue_t<T, DT_I8>(p, tc, acc, li); return; }
   }
-  if constexpr (T::DT == DT_FP8) {
+  if constexpr (is_f8(T::DT)) {
     if (p.c_type == DT_FP8) { epilogue_t<T, DT_FP8>(p, tc, acc, li); return; }
   }
   if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);

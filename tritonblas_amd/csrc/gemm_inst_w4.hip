@@ -1,10 +1,11 @@
-// The hand-scheduled 4-wave 256x256 kernels (FP8, MXFP4, bf16, fp16, int8), see gemm_w4.h.
+// The hand-scheduled 4-wave 256x256 kernels (FP8 e4m3 and e5m2, MXFP4, bf16, fp16, int8), see gemm_w4.h.
 #include "gemm_w4.h"
 
 namespace tb {
 
 const void* w4_kernel(int dt) {
   if (dt == DT_FP8) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP8>>;
+  if (dt == DT_E5M2) return (const void*)&gemm_kernel_w4<W4Tile<DT_E5M2>>;
   if (dt == DT_FP4) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP4>>;
   if (dt == DT_BF16) return (const void*)&gemm_kernel_w4<W4Tile<DT_BF16>>;
   if (dt == DT_F16) return (const void*)&gemm_kernel_w4<W4Tile<DT_F16>>;

@@ -43,6 +43,8 @@ extern const Variant g_variants_bf16[];
 extern const int g_num_variants_bf16;
 extern const Variant g_variants_fp8[];
 extern const int g_num_variants_fp8;
+extern const Variant g_variants_e5m2[];
+extern const int g_num_variants_e5m2;
 extern const Variant g_variants_fp4[];
 extern const int g_num_variants_fp4;
 extern const Variant g_variants_f32[];

@@ -240,7 +240,7 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
-  static_assert(T::DT == DT_FP8 || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16 || T::DT == DT_I8, "element types with a generated K loop");
+  static_assert(is_f8(T::DT) || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16 || T::DT == DT_I8, "element types with a generated K loop");
   // two stages, the FP4 scale buffers (16 KB), 1 KB per wave for epilogue scales, the schedule's broadcast word
   __shared__ __attribute__((aligned(16))) uint8_t lds[W4_LDS_BYTES];
   int& s_bcast = *(int*)(lds + W4_LDS_BYTES - 16);
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   int fe = 0;                       // 1: the previous tile's sums are still in the accumulators
   const uint8_t* cprev = (const uint8_t*)p.C;   // C[first row of the wave's quarter][its first column] of that tile
   const bool fe_shape = p.c_line && !p.bias && p.c_type == DT_BF16 && p.c_sm < (1 << 26) && (p.debug & 4) == 0 &&
-                        ((T::DT == DT_FP8 || T::DT == DT_I8) == (p.sa != nullptr));
+                        ((is_f8(T::DT) || T::DT == DT_I8) == (p.sa != nullptr));
   // a lane's C offset from cprev, the same in every row block (rows of a row block are c_sm apart);
   // lane * 4; where the lane finds the scales of its rows 16 i + r and of its columns 32 q + 8 g + 0..7
   v4i eo;
@@ -319,12 +319,12 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     w4_tile_args<T>(p, wnext.tc, ln, nxt);
     const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
                       (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
-    const bool regs = (T::DT == DT_FP8 || T::DT == DT_I8) && fast && p.sa;    // the K loop copies this tile's scale vectors
+    const bool regs = (is_f8(T::DT) || T::DT == DT_I8) && fast && p.sa;    // the K loop copies this tile's scale vectors
     const uint8_t *sA = uniform(cur.A), *sB = uniform(cur.B), *sAn = uniform(nxt.A), *sBn = uniform(nxt.B);
     const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst), s_fe = uniform(fe);
     const uint8_t* s_cprev = uniform(cprev);
     scbuf = uniform(scbuf);
-    if constexpr (T::DT == DT_FP8 || T::DT == DT_I8) {
+    if constexpr (is_f8(T::DT) || T::DT == DT_I8) {
       // (a tile without scales or off the fast path loads 512 bytes of its operands instead; nobody uses them)
       const uint8_t* s_sap = uniform(regs ? (const uint8_t*)(p.sa + w.tc.m0 + ln.wm0) : cur.A);
       const uint8_t* s_sbp = uniform(regs ? (const uint8_t*)(w.tc.sb + w.tc.n0 + ln.wn0) : cur.B);
@@ -335,6 +335,14 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
             : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
             :
 #include "w4_clobbers_fp8.inc"
+        );
+      } else if constexpr (T::DT == DT_E5M2) {
+        asm volatile(
+#include "w4_kloop_e5m2.inc"
+            : [scbuf] "+s"(scbuf)
+            : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
+            :
+#include "w4_clobbers_e5m2.inc"
         );
       } else {
         asm volatile(

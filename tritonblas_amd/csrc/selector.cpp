@@ -12,7 +12,7 @@ namespace tb {
 static int type_bits(int t) {
   switch (t) {
     case TB_F16: case TB_BF16: return 16;
-    case TB_FP8_E4M3: case TB_I8: return 8;
+    case TB_FP8_E4M3: case TB_FP8_E5M2: case TB_I8: return 8;
     case TB_FP4_E2M1: return 4;
     case TB_F32: return 32;
   }
@@ -23,7 +23,7 @@ static int type_bits(int t) {
 static double mfma_flops_per_clk(int t) {
   switch (t) {
     case TB_F16: case TB_BF16: return 4096.0;
-    case TB_FP8_E4M3: case TB_I8: return 8192.0;
+    case TB_FP8_E4M3: case TB_FP8_E5M2: case TB_I8: return 8192.0;
     case TB_FP4_E2M1: return 16384.0;
     case TB_F32: return 256.0;
   }
@@ -82,7 +82,7 @@ static double family_efficiency(int dt, const TileInfo& v) {
   static const double h16[4] = {0.59, 0.465, 0.22, 0.12};  // (128x128: 8192^3 bf16 in 0.97 ms)
   static const double f4[4] = {0.50, 0.36, 0.22, 0.10};     // (256x256: the 4-wave kernel, 8192x8192x16384 in 0.43-0.47 ms)
   static const double f32[4] = {0.80, 0.75, 0.60, 0.30};   // the fp32 matrix pipe is slow enough to hide everything else
-  if (dt == TB_FP8_E4M3 || dt == TB_I8) return f8[cls];
+  if (dt == TB_FP8_E4M3 || dt == TB_FP8_E5M2 || dt == TB_I8) return f8[cls];
   if (dt == TB_FP4_E2M1) return f4[cls];
   if (dt == TB_F32) return f32[cls];
   return h16[cls];
@@ -145,7 +145,7 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   // the 64x64 tile of the 8- and 16-bit float types runs with four (three) copy stages while no more
   // than two (three) tiles per CU exist, which hides that much more of the round trip (measured x0.67 / x0.85)
   if (v.bm == 64 && v.bn == 64 && pr.num_groups == 0 &&
-      (pr.a_type == TB_F16 || pr.a_type == TB_BF16 || pr.a_type == TB_FP8_E4M3)) {
+      (pr.a_type == TB_F16 || pr.a_type == TB_BF16 || pr.a_type == TB_FP8_E4M3 || pr.a_type == TB_FP8_E5M2)) {
     const int64_t whole = cdiv(pr.m, v.bm) * cdiv(pr.n, v.bn);
     if (whole <= 2 * (int64_t)hw.n_cu) t_lat *= 0.67;
     else if (whole <= 3 * (int64_t)hw.n_cu) t_lat *= 0.85;

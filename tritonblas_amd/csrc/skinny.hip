@@ -14,11 +14,11 @@
 namespace tb {
 
 template <int DT> struct SkT {
-  static constexpr int LB = (DT == DT_FP8) ? 32 : 16;   // bytes of K one lane feeds to one MFMA
+  static constexpr int LB = is_f8(DT) ? 32 : 16;        // bytes of K one lane feeds to one MFMA
   static constexpr int STEP = 4 * LB;                   // bytes of K per MFMA
-  using frag_t = typename std::conditional<DT == DT_FP8, v8i, v4i>::type;
+  using frag_t = typename std::conditional<is_f8(DT), v8i, v4i>::type;
   __device__ static __forceinline__ frag_t load(const uint8_t* p) {
-    if constexpr (DT == DT_FP8) {
+    if constexpr (is_f8(DT)) {
       v4i lo = *(const v4i*)p, hi = *(const v4i*)(p + 16);
       return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     } else {
@@ -28,7 +28,10 @@ template <int DT> struct SkT {
   __device__ static __forceinline__ v4f mma(frag_t x, frag_t y, v4f c) {
     if constexpr (DT == DT_F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, x), __builtin_bit_cast(h8, y), c, 0, 0, 0);
     else if constexpr (DT == DT_BF16) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, x), __builtin_bit_cast(bf8, y), c, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
+    else {
+      constexpr int FMT = DT == DT_E5M2 ? 1 : 0;   // 0 = e4m3, 1 = e5m2, both operands
+      return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, FMT, FMT, 0, 0, 0, 0);
+    }
   }
 };
 
@@ -40,7 +43,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_kernel(const GemmParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (16 * NT);
-  constexpr int USZ = (DT == DT_FP8) ? 1 : 2;
+  constexpr int USZ = is_f8(DT) ? 1 : 2;
 
   // this wave's share of the K steps
   const int64_t kbytes = p.KU * USZ;
@@ -145,12 +148,13 @@ static hipError_t launch_dt(const GemmParams& p, hipStream_t stream) {
   return launch_mt<DT, 4>(p, stream);
 }
 
-bool skinny_supported(int dt, int64_t m) { return m <= SKINNY_MAX_M && (dt == DT_FP8 || dt == DT_F16 || dt == DT_BF16); }
+bool skinny_supported(int dt, int64_t m) { return m <= SKINNY_MAX_M && (is_f8(dt) || dt == DT_F16 || dt == DT_BF16); }
 
-int skinny_k_step_units(int dt) { return dt == DT_FP8 ? 128 : 32; }
+int skinny_k_step_units(int dt) { return is_f8(dt) ? 128 : 32; }
 
 hipError_t launch_skinny(const GemmParams& p, int dt, hipStream_t stream) {
   if (dt == DT_FP8) return launch_dt<DT_FP8>(p, stream);
+  if (dt == DT_E5M2) return launch_dt<DT_E5M2>(p, stream);
   if (dt == DT_F16) return launch_dt<DT_F16>(p, stream);
   return launch_dt<DT_BF16>(p, stream);
 }

@@ -15,6 +15,10 @@
 
 using namespace tb;
 
+// the public element type codes are the kernels' own
+static_assert(TB_F16 == DT_F16 && TB_BF16 == DT_BF16 && TB_FP8_E4M3 == DT_FP8 && TB_FP4_E2M1 == DT_FP4 && TB_F32 == DT_F32 &&
+              TB_I8 == DT_I8 && TB_FP8_E5M2 == DT_E5M2, "element type codes");
+
 namespace {
 
 constexpr int MAX_DEVICES = 64;
@@ -112,6 +116,7 @@ void variant_table(int dt, const Variant** v, int* n) {
     case TB_F16: *v = g_variants_f16; *n = g_num_variants_f16; break;
     case TB_BF16: *v = g_variants_bf16; *n = g_num_variants_bf16; break;
     case TB_FP8_E4M3: *v = g_variants_fp8; *n = g_num_variants_fp8; break;
+    case TB_FP8_E5M2: *v = g_variants_e5m2; *n = g_num_variants_e5m2; break;
     case TB_FP4_E2M1: *v = g_variants_fp4; *n = g_num_variants_fp4; break;
     case TB_F32: *v = g_variants_f32; *n = g_num_variants_f32; break;
     case TB_I8: *v = g_variants_i8; *n = g_num_variants_i8; break;
@@ -230,7 +235,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
   if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
   if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8) &&
-      !(j.c_type == TB_FP8_E4M3 && j.dt == TB_FP8_E4M3))
+      !(j.c_type == TB_FP8_E4M3 && (j.dt == TB_FP8_E4M3 || j.dt == TB_FP8_E5M2)))
     return TB_ERR_BAD_DTYPE;
   const int usz = unit_bytes(j.dt);
   const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
@@ -667,7 +672,9 @@ int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
   if (d->a_type != d->b_type) return TB_ERR_BAD_DTYPE;
-  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_F32 && d->a_type != TB_I8) return TB_ERR_BAD_DTYPE;
+  if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_FP8_E5M2 && d->a_type != TB_F32 &&
+      d->a_type != TB_I8)
+    return TB_ERR_BAD_DTYPE;
   if ((d->a_scale == nullptr) != (d->b_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
   if (d->bias && d->bias_type != TB_F16 && d->bias_type != TB_BF16 && d->bias_type != TB_F32) return TB_ERR_BAD_DTYPE;
   j->dt = d->a_type; j->c_type = d->c_type; j->bias_type = d->bias_type;
