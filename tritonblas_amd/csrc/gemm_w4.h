@@ -282,9 +282,14 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   sched.init(p);
 #ifdef W4_LAB_STAGGER
   {
-    // measurement build: delay the start of workgroups by (id / div) % mod microseconds (debug = div*1000 + mod*... )
-    const int unit = p.debug / 10000, div = (p.debug / 100) % 100, mod = p.debug % 100;
-    if (mod > 0) { const int n = ((int)blockIdx.x / max(div, 1)) % mod * unit; for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(32); }
+    // measurement build: groups of the workgroups of one XCD (local index b / 8; its low three bits are the
+    // tile's row within the XCD's 8 x 4 block of tiles, the next two its column) start (debug >> 8) * 256
+    // cycles apart: debug & 3 = 1: two groups (rows 0..3 / 4..7), 2: four groups of two rows, 3: four
+    // groups, one per column
+    const int local = (int)blockIdx.x >> 3, mode = p.debug & 3;
+    const int grp = mode == 1 ? ((local >> 2) & 1) : mode == 2 ? ((local >> 1) & 3) : mode == 3 ? ((local >> 3) & 3) : 0;
+    const int n = grp * (p.debug >> 8);
+    for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);
   }
 #endif
   Work w, wnext;
