@@ -48,6 +48,7 @@ def test_driver_runs_a_shape_list_with_correctness_check(tmp_path, flags):
         {"m": 256, "n": 512, "k": 1024, "in_dtype": "bfloat16", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
         {"m": 300, "n": 200, "k": 512, "in_dtype": "float16", "out_dtype": "float16", "transA": "T", "transB": "T"},
         {"m": 512, "n": 256, "k": 2048, "in_dtype": "float8_e4m3fn", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
+        {"m": 256, "n": 512, "k": 1024, "in_dtype": "float8_e5m2", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
         {"m": 384, "n": 256, "k": 1024, "in_dtype": "int8", "out_dtype": "bfloat16", "transA": "T", "transB": "N"},
         {"m": 256, "n": 384, "k": 512, "in_dtype": "int8", "out_dtype": "int8", "transA": "T", "transB": "N"},
         {"m": 320, "n": 256, "k": 768, "in_dtype": "float32", "out_dtype": "float32", "transA": "T", "transB": "T"},

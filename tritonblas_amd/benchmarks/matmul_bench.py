@@ -35,13 +35,13 @@ FIELDNAMES = ["m", "n", "k", "mnk", "macro_tile", "bytes", "flops", "tritonblas_
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "float16": torch.float16, "fp16": torch.float16,
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float8_e4m3fn": torch.float8_e4m3fn,
-           "fp8": torch.float8_e4m3fn, "int8": torch.int8, "fp4": "fp4"}
+           "fp8": torch.float8_e4m3fn, "float8_e5m2": torch.float8_e5m2, "bf8": torch.float8_e5m2, "int8": torch.int8, "fp4": "fp4"}
 
 
 def str_to_dtype(name):
     key = str(name).replace("torch.", "").lower()
     if key not in _DTYPES:
-        raise ValueError(f"unsupported dtype {name!r}; this library runs float32, float16, bfloat16, float8_e4m3fn, int8 and fp4 inputs")
+        raise ValueError(f"unsupported dtype {name!r}; this library runs float32, float16, bfloat16, float8_e4m3fn, float8_e5m2, int8 and fp4 inputs")
     return _DTYPES[key]
 
 
