@@ -391,3 +391,14 @@ def test_library_hierarchical_split(total, hw_cus, xcds):
         assert (l.value, g.value) == (total // xcds, total - xcds * (total // xcds))
     assert lib.tb_hierarchical_split(0, hw_cus, xcds, C.byref(l), C.byref(g)) == -10
     assert lib.tb_hierarchical_split(total, hw_cus, xcds, None, C.byref(g)) == -1
+
+
+def test_grouped_gemm_refuses_other_operand_types():
+    """the grouped entry point computes in FP8 e4m3 whatever it is handed: other types must not be read as that"""
+    import tritonblas_amd as tb
+    a = torch.zeros(8, 128, dtype=torch.float8_e5m2)
+    w = torch.zeros(2, 16, 128, dtype=torch.float8_e5m2)
+    c = torch.zeros(8, 16, dtype=torch.bfloat16)
+    offs = torch.tensor([0, 4, 8], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+        tb.grouped_matmul_a8w8(a, w, None, None, c, offs)

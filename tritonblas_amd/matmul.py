@@ -388,6 +388,8 @@ def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int =
     E, N, K2 = w.shape
     assert K == K2 and c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
     assert group_offsets.numel() == E + 1 and group_offsets.dtype == torch.int32
+    if a.dtype != torch.float8_e4m3fn or w.dtype != torch.float8_e4m3fn:
+        raise RuntimeError(f"tritonblas_amd: grouped GEMM takes float8_e4m3fn operands, got {a.dtype} and {w.dtype}")
     dev = _check_device(a, w, c, a_scale, w_scale, group_offsets)
     if a.stride(1) != 1 or w.stride(2) != 1:
         raise RuntimeError("tritonblas_amd: grouped GEMM needs K-contiguous operands")
