@@ -402,3 +402,14 @@ def test_grouped_gemm_refuses_other_operand_types():
     offs = torch.tensor([0, 4, 8], dtype=torch.int32)
     with pytest.raises(RuntimeError, match="float8_e4m3fn"):
         tb.grouped_matmul_a8w8(a, w, None, None, c, offs)
+
+
+def test_matmul_fp4_refuses_wrong_element_sizes_and_scale_shapes():
+    import tritonblas_amd as tb
+    a, b = torch.zeros(8, 64, dtype=torch.uint8), torch.zeros(16, 64, dtype=torch.uint8)
+    c = torch.zeros(8, 16, dtype=torch.bfloat16)
+    sa, sb = torch.zeros(8, 4, dtype=torch.uint8), torch.zeros(16, 4, dtype=torch.uint8)
+    with pytest.raises(RuntimeError, match="one-byte"):
+        tb.matmul_fp4(a.to(torch.bfloat16), b, c, sa, sb)
+    with pytest.raises(RuntimeError, match="scales must be"):
+        tb.matmul_fp4(a, b, c, sa.T.contiguous(), sb)

@@ -353,6 +353,11 @@ def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = 
     N = b.shape[0]
     K = Kp * 2
     assert b.shape[1] * 2 == K, f"Incompatible Dimensions: A has K={K}, B has K={b.shape[1] * 2}"
+    for t in (a, b, a_scales, b_scales):
+        if t.element_size() != 1:
+            raise RuntimeError(f"tritonblas_amd: matmul_fp4 takes packed codes and E8M0 scales as one-byte elements, got {t.dtype}")
+    if tuple(a_scales.shape) != (M, K // 32) or tuple(b_scales.shape) != (N, K // 32):
+        raise RuntimeError(f"tritonblas_amd: matmul_fp4 scales must be (M, K/32) and (N, K/32), got {tuple(a_scales.shape)} and {tuple(b_scales.shape)}")
     dev = _check_device(a, b, c, a_scales, b_scales)
     a, b = a.view(torch.uint8), b.view(torch.uint8)
     a_scales, b_scales = a_scales.view(torch.uint8), b_scales.view(torch.uint8)
