@@ -153,6 +153,19 @@ def test_addmm_column_bias(m, n, k, dtype):
     _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32, bias=bias_cpu), dtype, TOL_16)
 
 
+def test_addmm_row_vector_bias_and_lone_scale():
+    """a (1, N) bias is one value per column like an (N,) one; a scale vector without its partner is refused"""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import persistent_matmul_lt
+    m, n, k = 64, 192, 256
+    a_cpu, b_cpu, bias_cpu = _rand((m, k), torch.bfloat16, 5, 0.5), _rand((k, n), torch.bfloat16, 6, 0.5), _rand((n,), torch.bfloat16, 7)
+    c = tb.addmm(bias_cpu.cuda().reshape(1, n), a_cpu.cuda(), b_cpu.cuda())
+    _check(c.cpu(), OG.ref_gemm(a_cpu, b_cpu, torch.float32, bias=bias_cpu), torch.bfloat16, TOL_16)
+    sel = tb.OrigamiMatmulSelector(m, n, k, torch.bfloat16, torch.bfloat16, torch.bfloat16, torch.device("cuda"))
+    with pytest.raises(RuntimeError, match="come together"):
+        persistent_matmul_lt(a_cpu.cuda(), b_cpu.cuda(), c, sel, None, a_scale=torch.ones(m, device="cuda"), quantized=True)
+
+
 # ---- FP8 a8w8 -----------------------------------------------------------------------------------
 def _a8w8_case(m, n, k, seed=2):
     g = torch.Generator().manual_seed(seed)

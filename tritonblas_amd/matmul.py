@@ -99,6 +99,8 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
     d.b_stride_k, d.b_stride_n = b.stride(0), b.stride(1)
     d.c_stride_m, d.c_stride_n = c.stride(0), c.stride(1)
     d.a, d.b, d.c = _ptr(a), _ptr(b), _ptr(c)
+    if (a_scale is None) != (b_scale is None):
+        raise RuntimeError("tritonblas_amd: a_scale and b_scale come together")
     if a_scale is not None:
         if a_scale.dtype != torch.float32 or b_scale.dtype != torch.float32:
             raise RuntimeError("tritonblas_amd: scales must be float32")
@@ -109,6 +111,8 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
     if bias is not None:
         if bias.numel() != N:
             raise AssertionError("Incompatible Dimensions")
+        if bias.dim() != 1:
+            bias = bias.reshape(-1)     # (1, N) and the like: one value per output column
         d.bias, d.bias_type, d.bias_stride = _ptr(bias), _lib.tb_dtype(bias.dtype), bias.stride(0)
     if selector is not None:
         d.block_m, d.block_n, d.block_k = selector.block_m, selector.block_n, selector.block_k
@@ -275,6 +279,7 @@ def _addmm_setup_context(ctx, inputs, output):
     bias, a, b, enable_streamk, sk_grid, work_stealing = inputs
     ctx.save_for_backward(a, b)
     ctx.opts = (enable_streamk, sk_grid, work_stealing)
+    ctx.bias_shape = tuple(bias.shape)
 
 
 def _addmm_backward(ctx, grad_output):
@@ -283,7 +288,7 @@ def _addmm_backward(ctx, grad_output):
     g = grad_output.contiguous()
     grad_a = matmul(g, b.T.contiguous(), enable_streamk=sk, sk_grid=grid, work_stealing=ws)
     grad_b = matmul(a.T.contiguous(), g, enable_streamk=sk, sk_grid=grid, work_stealing=ws)
-    return grad_output.sum(dim=0), grad_a, grad_b, None, None, None
+    return grad_output.sum(dim=0).reshape(ctx.bias_shape), grad_a, grad_b, None, None, None
 
 
 _addmm.register_autograd(_addmm_backward, setup_context=_addmm_setup_context)
