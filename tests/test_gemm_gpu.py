@@ -166,6 +166,21 @@ def test_addmm_row_vector_bias_and_lone_scale():
         persistent_matmul_lt(a_cpu.cuda(), b_cpu.cuda(), c, sel, None, a_scale=torch.ones(m, device="cuda"), quantized=True)
 
 
+def test_empty_operands():
+    """M, N or K of zero: nothing to compute, an untouched or zero-filled (plus bias) result as torch.matmul gives"""
+    import tritonblas_amd as tb
+    dev = torch.device("cuda")
+    for m, n, k in ((0, 64, 128), (64, 0, 128)):
+        a, b = torch.zeros(m, k, dtype=torch.bfloat16, device=dev), torch.zeros(k, n, dtype=torch.bfloat16, device=dev)
+        assert tb.matmul(a, b).shape == (m, n)
+    a, b = torch.zeros(32, 0, dtype=torch.bfloat16, device=dev), torch.zeros(0, 48, dtype=torch.bfloat16, device=dev)
+    c = torch.full((32, 48), float("nan"), dtype=torch.bfloat16, device=dev)
+    tb.matmul(a, b, out=c)
+    assert torch.equal(c, torch.zeros_like(c))
+    bias = torch.arange(48, dtype=torch.bfloat16, device=dev)
+    assert torch.equal(tb.addmm(bias, a, b), bias.expand(32, 48))
+
+
 # ---- FP8 a8w8 -----------------------------------------------------------------------------------
 def _a8w8_case(m, n, k, seed=2):
     g = torch.Generator().manual_seed(seed)

@@ -84,12 +84,28 @@ def _check_device(*tensors):
     return dev
 
 
+def _empty_problem(M, N, K, c, bias=None) -> bool:
+    """M, N or K of zero: torch.matmul's answer (nothing to write, or an empty sum = zeros plus the bias)
+    without a launch.  True when the problem was such a one."""
+    if M == 0 or N == 0:
+        return True
+    if K == 0:
+        if bias is None:
+            c.zero_()
+        else:
+            c.copy_(bias.reshape(1, N).to(torch.float32).expand(M, N))
+        return True
+    return False
+
+
 def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b_scale=None, sk_grid=None):
     assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
     M, K = a.shape
     _, N = b.shape
     assert c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
     dev = _check_device(a, b, c, bias, a_scale, b_scale)
+    if _empty_problem(M, N, K, c, bias):
+        return c
     lib = _lib.load()
     d = _lib.tb_gemm_desc()
     d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
@@ -197,6 +213,8 @@ def matmul_a8w8_lt(a, b, a_scale, b_scale, c, selector, config: MatmulConfig = N
 def _run(a, b, out, bias, enable_streamk, sk_grid, work_stealing, out_dtype_for_selector):
     M, K = a.shape
     _, N = b.shape
+    if _empty_problem(M, N, K, out, bias):
+        return out
     selector = _make_matmul_selector(M, N, K, a.dtype, b.dtype, out_dtype_for_selector, a.device,
                                      streamk=bool(enable_streamk))
     config = matmul_preamble(selector, a.device) if work_stealing else None
@@ -340,6 +358,8 @@ def matmul_a8w8(a, b, a_scale, b_scale, c, enable_streamk=False, work_stealing=F
     assert a.shape[1] == b.shape[0], "Incompatible Dimensions"
     M, K = a.shape
     _, N = b.shape
+    if _empty_problem(M, N, K, c):
+        return c
     selector = _make_matmul_selector(M, N, K, a.dtype, b.dtype, c.dtype, a.device, streamk=bool(enable_streamk))
     config = matmul_preamble(selector, a.device) if work_stealing else None
     if enable_streamk:
@@ -364,6 +384,8 @@ def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = 
     if tuple(a_scales.shape) != (M, K // 32) or tuple(b_scales.shape) != (N, K // 32):
         raise RuntimeError(f"tritonblas_amd: matmul_fp4 scales must be (M, K/32) and (N, K/32), got {tuple(a_scales.shape)} and {tuple(b_scales.shape)}")
     dev = _check_device(a, b, c, a_scales, b_scales)
+    if M == 0 or N == 0:
+        return c
     a, b = a.view(torch.uint8), b.view(torch.uint8)
     a_scales, b_scales = a_scales.view(torch.uint8), b_scales.view(torch.uint8)
     if a.stride(1) != 1 or b.stride(1) != 1:
@@ -401,6 +423,8 @@ def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int =
     if a.dtype != torch.float8_e4m3fn or w.dtype != torch.float8_e4m3fn:
         raise RuntimeError(f"tritonblas_amd: grouped GEMM takes float8_e4m3fn operands, got {a.dtype} and {w.dtype}")
     dev = _check_device(a, w, c, a_scale, w_scale, group_offsets)
+    if M == 0 or N == 0:
+        return c
     if a.stride(1) != 1 or w.stride(2) != 1:
         raise RuntimeError("tritonblas_amd: grouped GEMM needs K-contiguous operands")
     d = _lib.tb_grouped_gemm_desc()
