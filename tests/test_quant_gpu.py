@@ -109,6 +109,18 @@ def test_strided_rows():
     assert np.array_equal(codes.cpu().numpy(), want_c) and np.array_equal(scales.cpu().numpy(), want_s)
 
 
+def test_misaligned_view_and_empty_input():
+    """a view that starts off a 16-byte boundary (or whose rows do) is copied first; no rows: empty results"""
+    import tritonblas_amd as tb
+    x = torch.randn(40, 200, generator=torch.Generator().manual_seed(2)).bfloat16()
+    xs = x.cuda()[:, 3:3 + 160]          # starts 6 bytes into a row, row stride 400 bytes
+    codes, scales = tb.dynamic_mxfp4_quant(xs)
+    want_c, want_s = OM.mxfp4_quant(x[:, 3:3 + 160].float().numpy())
+    assert np.array_equal(codes.cpu().numpy(), want_c) and np.array_equal(scales.cpu().numpy(), want_s)
+    codes, scales = tb.hadamard_mxfp4_quant(torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda"))
+    assert codes.shape == (0, 32) and scales.shape == (0, 2)
+
+
 def test_quant_then_gemm_roundtrip():
     """Rotating both operands leaves A @ B^T unchanged: the MXFP4 GEMM of the two rotated+quantised
     operands approximates the bf16 product (quantisation noise only)."""

@@ -59,8 +59,8 @@ def _quant(x: torch.Tensor, hadamard: bool, out=None):
     assert N % 32 == 0, f"N ({N}) must be divisible by 32"
     if not x.is_cuda:
         raise RuntimeError("tritonblas_amd: the MXFP4 quantiser runs on the GPU only")
-    if x.stride(1) != 1:
-        x = x.contiguous()
+    if x.stride(1) != 1 or x.data_ptr() % 16 or (x.stride(0) * x.element_size()) % 16:
+        x = x.contiguous()      # (the kernel reads rows with 16-byte loads)
     if out is None:
         codes = torch.empty((M, N // 2), dtype=torch.uint8, device=x.device)
         scales = torch.empty((M, N // 32), dtype=torch.uint8, device=x.device)
@@ -69,6 +69,8 @@ def _quant(x: torch.Tensor, hadamard: bool, out=None):
         for t, cols in ((codes, N // 2), (scales, N // 32)):
             assert t.dtype == torch.uint8 and t.device == x.device and tuple(t.shape) == (M, cols) and t.stride(1) == 1, \
                 "out must be (codes (M, N/2), scales (M, N/32)) uint8 tensors on x's device with unit column stride"
+    if M == 0 or N == 0:
+        return codes, scales
     d = _lib.tb_quant_desc()
     d.struct_bytes = C.sizeof(_lib.tb_quant_desc)
     d.x_type = _lib.tb_dtype(x.dtype)
