@@ -14,3 +14,10 @@ const void* w4_kernel(int dt) {
 }
 
 }  // namespace tb
+
+#ifdef W4_LAB_TS
+// measurement build: copies the timestamps of the last launch to the host (synchronises)
+extern "C" int tb_lab_timestamps(unsigned long long* dst) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(tb::w4_lab_ts), sizeof(tb::w4_lab_ts));
+}
+#endif

@@ -237,6 +237,11 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
       [An] "s"(sAn), [Bn] "s"(sBn), [wl] "s"(wl), [kh] "s"(s_kh), [first] "s"(s_first), [nst] "s"(s_nst), [fe] "s"(s_fe), \
       [cprev] "s"(s_cprev), [cstep] "s"(s_cstep)
 
+#ifdef W4_LAB_TS
+// measurement build: when (constant 100 MHz counter) every workgroup started and finished each of its tiles
+__device__ unsigned long long w4_lab_ts[1024 * 32];
+#endif
+
 template <class T>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
@@ -291,6 +296,11 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     const int n = grp * (p.debug >> 8);
     for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);
   }
+#endif
+#ifdef W4_LAB_TS
+  int ts_n = 0;
+  if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
+  ++ts_n;
 #endif
   Work w, wnext;
   bool have = sched.next(p, w, &s_bcast, tid);
@@ -417,12 +427,19 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
       else epilogue_w4<T, DT_F32>(p, w.tc, ln);
       nst = fast ? 1 : 0;
     }
+#ifdef W4_LAB_TS
+    if (tid == 0 && blockIdx.x < 1024 && ts_n < 31) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
+    ++ts_n;
+#endif
     w.tc = wnext.tc;
     have = have_next;
     first = 0;
   }
   // the last tile's look-ahead copies still write LDS: they must have landed before the workgroup ends
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef W4_LAB_TS
+  if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + 31] = __builtin_amdgcn_s_memrealtime();
+#endif
   if (p.mode == MODE_WS && tid == 0) {
     // the last workgroup to leave rearms the queues for the next launch
     uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
