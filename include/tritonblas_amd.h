@@ -187,6 +187,12 @@ size_t tb_workspace_bytes(const tb_gemm_desc* desc);
 #define TB_EPOCH_ON_DEVICE 0xFFFFFFFFu
 int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream);
 
+/* Reads the status word of the current GPU's static workspace into *status (1: a Stream-K launch through
+ * tb_gemm_static_workspace ran into spin_limit and stored NaN tiles) and, with clear != 0, sets it back to 0.
+ * Waits for the device's earlier work; allocates nothing.  A caller-owned workspace carries the same word at
+ * byte 0 (MatmulConfig.status() / check(), config.py of this package).  No counterpart in the reference. */
+int tb_static_workspace_status(int* status, int clear);
+
 /* Byte offsets of the regions of a workspace: [0, 256) control words -- word 0 is the status (set to 1
  * when a Stream-K wait ran into spin_limit: the tile concerned was then stored as NaN; cleared only by the
  * caller), word 1 counts workgroups that have finished (work stealing, and Stream-K with

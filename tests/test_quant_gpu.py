@@ -117,6 +117,13 @@ def test_misaligned_view_and_empty_input():
     codes, scales = tb.dynamic_mxfp4_quant(xs)
     want_c, want_s = OM.mxfp4_quant(x[:, 3:3 + 160].float().numpy())
     assert np.array_equal(codes.cpu().numpy(), want_c) and np.array_equal(scales.cpu().numpy(), want_s)
+    # a CONTIGUOUS view that merely starts two bytes off a 16-byte boundary
+    flat = torch.randn(1 + 24 * 128, generator=torch.Generator().manual_seed(3)).bfloat16()
+    xv = flat.cuda()[1:].view(24, 128)
+    assert xv.is_contiguous() and xv.data_ptr() % 16 == 2
+    codes, scales = tb.dynamic_mxfp4_quant(xv)
+    want_c, want_s = OM.mxfp4_quant(flat[1:].view(24, 128).float().numpy())
+    assert np.array_equal(codes.cpu().numpy(), want_c) and np.array_equal(scales.cpu().numpy(), want_s)
     codes, scales = tb.hadamard_mxfp4_quant(torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda"))
     assert codes.shape == (0, 32) and scales.shape == (0, 2)
 

@@ -335,7 +335,65 @@ def test_streamk_poll_bound_poisons_the_tile():
     cfg.check()
 
 
+def test_streamk_poll_bound_two_tiles_one_workgroup():
+    """Three workgroups share four tiles: the last workgroup owns a whole tile (no partner) and the tail of the
+    tile before it (partner: workgroup 1).  With a poll bound of one, whatever it could not finish is NaN and
+    everything else is right -- no tile of a workgroup that gave up is left as stale memory -- and with an e4m3
+    result the poisoned tile reads as NaN bytes, not as a clamped finite value."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    m, n, k = 512, 512, 8192
+    aq, bq, sa, sb = _fp8_case(m, n, k, 83)
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    for out_dtype in (torch.bfloat16, torch.float8_e4m3fn):
+        want = OG.ref_gemm(aq, bq, out_dtype, a_scale=sa, b_scale=sb).float()
+        sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, out_dtype, a.device, streamk=True)
+        sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 128
+        cfg = tb.matmul_preamble(sel)
+        cfg.ensure(64 << 20)
+        cfg.spin_limit = 1
+        c = torch.full((m, n), 7.0, device="cuda").to(out_dtype)
+        streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=3, a_scale=sa.cuda(), b_scale=sb.cuda(), quantized=True)
+        torch.cuda.synchronize()
+        got = c.float().cpu()
+        failed = cfg.status() != 0
+        assert failed == bool(torch.isnan(got).any()), "NaN tiles and the status word go together"
+        ok = ~torch.isnan(got)
+        # (whole 256x256 tiles are poisoned, nothing else; no 7.0 of the initial fill survives anywhere)
+        for ti in range(2):
+            for tj in range(2):
+                blk = ok[ti * 256:(ti + 1) * 256, tj * 256:(tj + 1) * 256]
+                assert blk.all() or not blk.any()
+        if out_dtype == torch.bfloat16:
+            assert OG.rel_fro_error(got[ok], want[ok]) <= 1e-2
+        else:
+            torch.testing.assert_close(got[ok], want[ok], atol=2.0, rtol=0.2)
+        cfg.clear_status()
+
+
 # ---- e4m3 output ---------------------------------------------------------------------------------------------
+def test_a8w8_fp8_output_keeps_nan():
+    """torch.clamp keeps NaN (the reference's oracle, tests/test_matmul_a8w8_lt.py:11-38): a row whose scale is
+    NaN must come out as e4m3 NaN bytes, a row whose scale is +Inf as +-448 (or NaN where the sum is zero)."""
+    import tritonblas_amd as tb
+    m, n, k = 256, 512, 512
+    aq, bq, sa, sb = _fp8_case(m, n, k, 92)
+    sa = sa.clone()
+    sa[3] = float("nan")
+    sa[100] = float("inf")
+    a, b = aq.cuda(), bq.T.contiguous().cuda().T
+    for streamk in (False, True):
+        c = torch.zeros(m, n, dtype=torch.float8_e4m3fn, device="cuda")
+        tb.matmul_a8w8(a, b, sa.cuda(), sb.cuda(), c, enable_streamk=streamk)
+        want = OG.ref_gemm(aq, bq, torch.float8_e4m3fn, a_scale=sa, b_scale=sb).float()
+        got = c.float().cpu()
+        assert torch.isnan(want[3]).all() and torch.isnan(got[3]).all()
+        assert torch.equal(torch.isnan(got), torch.isnan(want))
+        assert torch.equal(got[100][~torch.isnan(got[100])], want[100][~torch.isnan(want[100])])
+        fin = ~torch.isnan(want)
+        torch.testing.assert_close(got[fin], want[fin], atol=2.0, rtol=0.2)
+
+
 @pytest.mark.parametrize("m,n,k", [(256, 256, 256), (100, 300, 640), (512, 1024, 512)])
 @pytest.mark.parametrize("streamk", [False, True])
 def test_a8w8_fp8_output(m, n, k, streamk):

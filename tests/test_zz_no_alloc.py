@@ -63,3 +63,34 @@ def test_static_workspace_rejects_what_does_not_fit():
     d.block_m, d.block_n, d.block_k = 256, 256, 64
     assert lib.tb_workspace_bytes(d) > 16 << 20
     assert lib.tb_gemm_static_workspace(d, _lib.stream_handle()) == _lib.TB_ERR_WORKSPACE
+
+
+def test_static_workspace_status_word():
+    """tb_static_workspace_status reads (and clears) the status word a poll-bound Stream-K launch sets in the
+    library's own array.  The bound is forced from the host (one poll); every kernel still ends normally."""
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    st = C.c_int(-1)
+    assert lib.tb_static_workspace_status(C.byref(st), 1) == _lib.TB_OK
+    assert lib.tb_static_workspace_status(C.byref(st), 0) == _lib.TB_OK and st.value == 0
+    assert lib.tb_static_workspace_status(None, 0) == _lib.TB_ERR_NULL_POINTER
+    m, n, k = 256, 256, 8192
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = (torch.randn(m, k, device="cuda", generator=g) * 0.5).bfloat16()
+    b = (torch.randn(k, n, device="cuda", generator=g) * 0.5).bfloat16()
+    c = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    d = _desc(_lib, a, b, c, _lib.TB_SCHED_STREAMK, 16)
+    d.block_m, d.block_n, d.block_k = 256, 256, 64
+    d.spin_limit = 1
+    assert lib.tb_gemm_static_workspace(d, _lib.stream_handle()) == _lib.TB_OK
+    assert lib.tb_static_workspace_status(C.byref(st), 0) == _lib.TB_OK
+    poisoned = bool(torch.isnan(c.float()).any())
+    assert (st.value != 0) == poisoned
+    assert lib.tb_static_workspace_status(C.byref(st), 1) == _lib.TB_OK
+    assert lib.tb_static_workspace_status(C.byref(st), 0) == _lib.TB_OK and st.value == 0
+    d.spin_limit = 0
+    assert lib.tb_gemm_static_workspace(d, _lib.stream_handle()) == _lib.TB_OK
+    torch.cuda.synchronize()
+    ref = (a.float() @ b.float()).bfloat16()
+    assert ((c.float() - ref.float()).norm() / ref.float().norm()).item() <= 1e-3
+    assert lib.tb_static_workspace_status(C.byref(st), 0) == _lib.TB_OK and st.value == 0

@@ -27,7 +27,7 @@ EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
     "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile", "tb_hierarchical_split",
-    "tb_workspace_layout", "tb_debug_option", "tb_gemm_static_workspace",
+    "tb_workspace_layout", "tb_debug_option", "tb_gemm_static_workspace", "tb_static_workspace_status",
 ]
 
 
@@ -123,6 +123,8 @@ def load():
     lib.tb_ws_queue_tile.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32)] * 2
     lib.tb_hierarchical_split.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.tb_gemm_static_workspace.argtypes = [C.POINTER(tb_gemm_desc), C.c_void_p]
+    lib.tb_static_workspace_status.argtypes = [C.POINTER(C.c_int), C.c_int]
+    lib.tb_static_workspace_status.restype = C.c_int
     lib.tb_workspace_layout.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
     lib.tb_debug_option.argtypes = [C.c_char_p, C.c_int]
     if lib.tb_abi_version() != 1:

@@ -40,6 +40,7 @@ class MatmulConfig:
         self.global_atomic = global_atomic
         self.hierarchical = hierarchical
         self.epoch = 0
+        self._retired = []      # outgrown workspaces (kept: a captured launch may still name them)
         self.spin_limit = 0     # Stream-K: polls per wait before an owner gives up (0: the library's 2**24)
 
     @property
@@ -56,8 +57,17 @@ class MatmulConfig:
         return self._mask if self._use_mask else None
 
     def ensure(self, nbytes: int):
-        """Grow the workspace to at least nbytes (zero-initialised)."""
+        """Grow the workspace to at least nbytes (zero-initialised).  A workspace that has been handed to a
+        launch is never freed: a launch captured into a HIP graph holds its raw pointer, so the buffers this
+        config outgrows stay alive with it (a captured graph pins its config).  Under stream capture nothing
+        may be allocated or cleared -- the fill would become a node of the graph -- so a call that would have
+        to grow the workspace there raises: make the first call outside the capture."""
         if self.workspace is None or self.workspace.numel() < nbytes:
+            if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("tritonblas_amd: this launch needs a larger workspace than its config holds, and "
+                                   "the stream is being captured; run the call once outside the capture first")
+            if self.workspace is not None:
+                self._retired.append(self.workspace)
             self.workspace = torch.zeros(int(nbytes), dtype=torch.uint8, device=self.device)
             self.epoch = 0
         return self.workspace

@@ -835,10 +835,12 @@ template <int CT>
 __device__ __forceinline__ void store4(uint8_t* C, int64_t off_el, int64_t sn, v4f v, int nvalid, bool vec) {
   if constexpr (CT == DT_FP8) {
     // fp32 -> e4m3fn: clamp to the largest finite value, then round to nearest even
-    // (the reference's a8w8 oracle, tests/test_matmul_a8w8_lt.py:11-38)
+    // (the reference's a8w8 oracle, tests/test_matmul_a8w8_lt.py:11-38).  torch.clamp keeps NaN, and so
+    // does this: fmaxf / fminf return their other argument for a NaN, which would turn a poisoned or
+    // overflowed-to-NaN result into a plausible -448.
     float c[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) c[j] = fminf(fmaxf(v[j], -448.f), 448.f);
+    for (int j = 0; j < 4; ++j) c[j] = (v[j] != v[j]) ? v[j] : fminf(fmaxf(v[j], -448.f), 448.f);
     int w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
     w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
     uint8_t* cp = C + off_el;
@@ -1346,7 +1348,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   Sched<T, SK> sched;
   sched.init(p);
   Work w;
-  bool failed = false;
+  bool failed = false;   // a Stream-K wait ran into its poll bound (the status word tells the host)
   // The tag of this launch's partial tiles: the caller's epoch, or one more than the count the
   // workspace keeps itself (control word CTL_EPOCH, which the last workgroup to leave advances) --
   // the form a launch replayed from a captured graph needs, whose arguments cannot change.
@@ -1354,7 +1356,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   if constexpr (SK) {
     if (p.epoch == EPOCH_ON_DEVICE) epoch = __hip_atomic_load(p.ctl + CTL_EPOCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
   }
-  while (!failed && sched.next(p, w, &s_bcast, li.tid)) {
+  while (sched.next(p, w, &s_bcast, li.tid)) {
     __syncthreads();  // the previous item's store staging may still be read by slower waves
     mainloop<T, !SK>(p, w.tc, w.it0, w.it1, acc, lds, li);
     if constexpr (SK) {
@@ -1398,7 +1400,8 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
           // a partner did not publish within the bound (the bound is too tight, or the device is shared
           // with something that starves it): the tile cannot
           // be finished.  It is stored as NaN so that nobody mistakes stale memory for a result, and the
-          // status word tells the host.
+          // status word tells the host.  The workgroup then goes on with the rest of its work list: every
+          // tile it owns ends up either finished or NaN, never untouched.
           failed = true;
           const float nanv = __builtin_nanf("");
 #pragma unroll

@@ -83,13 +83,8 @@ template <class T>
 __device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, W4TileArgs& t) {
   const int rva = tc.m_lim - tc.m0, rvb = tc.n_lim - tc.n0;
   const uint32_t sra = (uint32_t)p.a_sr * T::USZ, srb = (uint32_t)p.b_sr * T::USZ;   // row strides in bytes
-#ifdef W4_LAB_SAMETILE
-  t.A = p.A;   // measurement build: every tile reads the operands of tile (0, 0) (all copies hit in L2)
-  t.B = tc.B;
-#else
   t.A = p.A + (int64_t)tc.m0 * p.a_sr * T::USZ;
   t.B = tc.B + (int64_t)tc.n0 * p.b_sr * T::USZ;
-#endif
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     t.off[i] = (int)((uint32_t)min(i * 32 + ln.pa, rva - 1) * sra + ln.c16);
@@ -285,18 +280,6 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
 
   Sched<T, false> sched;
   sched.init(p);
-#ifdef W4_LAB_STAGGER
-  {
-    // measurement build: groups of the workgroups of one XCD (local index b / 8; its low three bits are the
-    // tile's row within the XCD's 8 x 4 block of tiles, the next two its column) start (debug >> 8) * 256
-    // cycles apart: debug & 3 = 1: two groups (rows 0..3 / 4..7), 2: four groups of two rows, 3: four
-    // groups, one per column
-    const int local = (int)blockIdx.x >> 3, mode = p.debug & 3;
-    const int grp = mode == 1 ? ((local >> 2) & 1) : mode == 2 ? ((local >> 1) & 3) : mode == 3 ? ((local >> 3) & 3) : 0;
-    const int n = grp * (p.debug >> 8);
-    for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(4);
-  }
-#endif
 #ifdef W4_LAB_TS
   int ts_n = 0;
   if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
@@ -409,11 +392,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
       // L2s take such a burst as ordinary write-back lines and drain it behind the next K steps, while
       // non-temporal stores go to the fabric at once and hold the waves at the store queue (measured:
       // FP8 8192x28672x8192 1.24 -> 1.20 ms, MXFP4 8192x8192x16384 0.440 -> 0.415 ms without the hint).
-#ifdef W4_LAB_NT
-      const bool c_nt = p.c_nt;
-#else
       const bool c_nt = false;
-#endif
       if (fast) {
         if (p.c_type == DT_BF16) {
           if (c_nt) epilogue_w4_fast<T, DT_BF16, true>(p, w.tc, ln);

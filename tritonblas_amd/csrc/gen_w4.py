@@ -62,6 +62,7 @@ Register map (VGPR):  0..127   B fragment sets 0/1 (8 fragments x 8 registers ea
 SGPR 70..89 are scratch (copy cursors, loop counter, scale buffer toggle, flags, C row pointer).
 """
 import os
+import re
 import sys
 
 STAGE = 65536
@@ -86,7 +87,10 @@ class WaitVm:
     unknown compiled stores, "d" fused epilogue, "s" steady state, "f" first even step after the first
     two) to n."""
     def __init__(self, awaits, vals):
-        self.awaits, self.vals = awaits, {k: min(63, v) for k, v in vals.items()}
+        # vals: {history: n}, or a list of histories whose n the generator works out by replay (Gen.solve)
+        if not isinstance(vals, dict):
+            vals = {k: None for k in vals}
+        self.awaits, self.vals = awaits, {k: (None if v is None else min(63, v)) for k, v in vals.items()}
 
 
 class Gen:
@@ -106,6 +110,12 @@ class Gen:
         # instruction out (noscale: the MXFP4 kernel's scale copies and scale reads) to time the rest; results are then meaningless.  dmaonce = nodma except for the
         # first tile's entry copies, so that the LDS holds real operand data for the MFMAs to chew on.
         self.lab = set(lab)
+        # earlyb: the B rows of fragments 0..3 (copied first) are published by the X of the step after the copy instead of
+        # its Y, and the next step's B fragments 0..3 are read between X and Y (the LDS is idle there and the stretch
+        # behind Y cannot take all the fragment reads); earlysc (MXFP4): the scale copy leads that group, so the next
+        # step's scale reads move in front of Y in every step, not only in those that stay inside a scale group
+        self.earlyb = os.environ.get("W4GEN_EARLYB", "1" if kind == "fp4" else "0") == "1"
+        self.earlysc = os.environ.get("W4GEN_EARLYSC", "0") == "1"
         self.v_coff = 238 if self.fp4 else 240
         self.v_lane4, self.v_sa_rd, self.v_sb_rd = 241, 242, 243
         self.v_sb, self.v_sa, self.epi_tmp = 64, 96, 104
@@ -247,40 +257,54 @@ class Gen:
         return out
 
     # ---- one K step -------------------------------------------------------------------------------
-    def step(self, p, nxt, prefetch, flavor="steady"):
+    def step(self, p, nxt, prefetch, flavor="steady", pending0=None):
         """K step in stage p (= B set p, scale set p).  nxt: the copies issued in this step read the
-        next tile.  prefetch: request the following step's fragments at the end.  flavor: "steady",
-        "first0" (step 0 of a tile), "first0_fe" (with the previous tile's epilogue fused in), "first1".
-        Group tags are relative to this step: ("X", 0), ("Y", 0), awaited ("Y", -2), ("X", -1)."""
+        next tile.  prefetch: request the following step's fragments.  flavor: "steady", "first0" (step 0
+        of a tile), "first0_fe" (with the previous tile's epilogue fused in), "first1".  Group tags are
+        relative to this step: ("XB", 0) / ("X", 0) / ("Y", 0) are issued, ("Y", -2) or ("XB", -1) and
+        ("X", -1) awaited.  pending0: the LDS reads that may still be in flight when the step starts
+        (oldest first, one set of destination registers each)."""
         nm = self.nm
         total = 8 * nm
         first0 = flavor in ("first0", "first0_fe")
         fe = flavor == "first0_fe"
+        eb = self.earlyb
+        # early: the next step's B fragments 0..3 (and E8M0 scales) are read between X and Y instead of behind Y
+        early = eb and prefetch and not fe
+        q = p ^ 1
         out = [Op(f"; ---- K step, stage {p}, {flavor}{' (copies: next tile)' if nxt else ''}{'' if prefetch else ' (last of the tile)'}")]
         pre = [[] for _ in range(total)]      # in front of MFMA slot m
         post = [[] for _ in range(total)]     # behind it
         ops = self.dma(p, nxt, None)
-        lo = [ops[i] for i in (0, 1, 4, 5)]                 # A rows of row blocks 0..3 (both wave rows)
-        hi = [ops[i] for i in (2, 3, 6, 7)]
-        ops_b = ops[8:]
-        for o in lo + ops_b:
-            o[-1].vm = ("X", 0)
-        for o in hi:
+        a_lo = [ops[i] for i in (0, 1, 4, 5)]                 # A rows of row blocks 0..3 (both wave rows)
+        a_hi = [ops[i] for i in (2, 3, 6, 7)]
+        b_lo = [ops[8 + i] for i in (0, 1, 4, 5)]             # B rows of fragments 0..3 (both wave columns)
+        b_hi = [ops[8 + i] for i in (2, 3, 6, 7)]
+        has_sc = self.fp4 and p == 0
+        if eb:
+            # what the next step's X waits for comes first
+            sc_head = has_sc and self.earlysc
+            sc = self.scale_dma(nxt, ("XB", 0) if sc_head else ("X", 0)) if has_sc else []
+            for o in b_lo:
+                o[-1].vm = ("XB", 0)
+            for o in b_hi + a_lo:
+                o[-1].vm = ("X", 0)
+            xops = (sc if sc_head else []) + b_lo + b_hi + a_lo + ([] if sc_head else sc)
+        else:
+            sc = self.scale_dma(nxt, ("X", 0)) if has_sc else []
+            for o in ops[8:] + a_lo:
+                o[-1].vm = ("X", 0)
+            xops = ops[8:] + a_lo + sc
+        for o in a_hi:
             o[-1].vm = ("Y", 0)
         adv = self.dma_advance()
         adv_a, adv_b = adv[:2], adv[2:]
-        sc = self.scale_dma(nxt, ("X", 0)) if (self.fp4 and p == 0) else []
-        nx = len(ops_b) + len(lo) + len(sc)                   # copies issued behind X of this step
-        nxo = 12 + (2 if (self.fp4 and p == 1) else 0)        # ... behind X of the neighbouring steps
         nsc = self.nsc
-        # fused epilogue: row block 0 in front of the first MFMA, row block i+1 between the MFMAs of row block i
-        n_st = [0] * (total + 1)   # stores issued in front of slot m
         if fe:
-            # row block 0 in front of the first MFMA, the others spread over row blocks 0..4: block k is
-            # done before slot 5 nm k / 7 <= nm k, where its accumulators are overwritten, and everything
-            # is done before the fragments of step 1 arrive in the registers used here
+            # fused epilogue: row block 0 in front of the first MFMA, the others spread over row blocks 0..4:
+            # block k is done before slot 5 nm k / 7 <= nm k, where its accumulators are overwritten, and
+            # everything is done before the fragments of step 1 arrive in the registers used here
             blocks = [self.epilogue_block(i, ("ST", 0)) for i in range(8)]
-            pre[0] += [Op("s_waitcnt lgkmcnt(15)")] if self.scaled_epi else []
             pre[0] += blocks[0]
             rest = [o for b in blocks[1:] for o in b]
             for n, o in enumerate(rest):
@@ -289,34 +313,16 @@ class Gen:
         if flavor == "first1" and nsc:
             pre[0] += self.scale_loads(("SC", 0))
         pre[0] += self.frag_read(self.vA(3), 0, p, 3)
-        pre[0].append(Op("s_waitcnt lgkmcnt(6)"))
         xs = nm + self.xoff
         tail0 = 5 * nm + self.yoff
-        if fe:
-            # (stores in program order in front of X and Y)
-            def stores_before(slot):
-                c = sum(1 for o in pre[0] if o.vm == ("ST", 0))
-                for m in range(slot):
-                    c += sum(1 for o in post[m] if o.vm == ("ST", 0))
-                return c
-            sx, sy = stores_before(xs), stores_before(tail0)
-        # X
-        if flavor == "steady":
-            if p == 0 and nsc:
-                wx = WaitVm(("Y", -2), {"s": nxo + 4, "f": nxo + 4 + nsc})
-            else:
-                wx = WaitVm(("Y", -2), {"s": nxo + 4})
-        elif flavor == "first0":
-            wx = WaitVm(("Y", -2), {"a": nxo + 4, "b": nxo + 4 + NST, "c": 0})
-        elif flavor == "first0_fe":
-            wx = WaitVm(("Y", -2), {"d": nxo + 4 + sx})
-        else:   # first1: the previous tile's stores (compiled or fused) are younger than the awaited copies
-            wx = WaitVm(("Y", -2), {"a": nxo + 4 + nsc, "b": nxo + 4 + nsc + NST, "c": nxo + 4 + nsc, "d": nxo + 4 + nsc + NST})
+        # X: history keys of the waits (the counts are worked out by replay, see solve)
+        keys = {"steady": ["s"], "first0": ["a", "b", "c"], "first0_fe": ["d"], "first1": ["a", "b", "c", "d"]}[flavor]
+        keys_x = ["s", "f"] if (flavor == "steady" and p == 0 and nsc) else keys
+        wx = WaitVm(("XB", -1) if early else ("Y", -2), keys_x)
         pre[xs] += [Op("s_waitcnt lgkmcnt(0)"), wx, Op("s_barrier")]
         if flavor == "steady" and p == 0 and nsc:
             post[xs].append(Op(f"s_mov_b32 s{S_AFTER}, 0"))
         pre[xs] += self.frag_read(self.vA(4), 0, p, 4)
-        xops = ops_b + lo + sc
         span = 5 * nm - 2 - xs
         m0_slots = set()
 
@@ -336,28 +342,31 @@ class Gen:
         pre[2 * nm] += self.frag_read(self.vA(5), 0, p, 5)
         pre[3 * nm] += self.frag_read(self.vA(6), 0, p, 6)
         pre[4 * nm] += self.frag_read(self.vA(7), 0, p, 7)
-        # (A fragment 4 was requested at X; fragments 5, 6, 7 are younger)
-        pre[4 * nm].append(Op("s_waitcnt lgkmcnt(6)"))
+        # the next step's scale group: (p == 1) it sits in the other buffer; it has been published by this
+        # step's X when its copy leads the X group of the step before, else by this step's Y
+        sc_early = early and self.fp4 and (p == 0 or self.earlysc)
+        sc_flip = [Op(f"v_xor_b32 v240, {SCBUF}, v240"), Op(f"v_xor_b32 v241, {SCBUF}, v241")] if (self.fp4 and p == 1 and prefetch) else []
+        if early:
+            er = []
+            for jb in range(4):
+                er += self.frag_read(self.vB(q, jb), 1, q, jb)
+            if sc_early:
+                post[xs] += sc_flip
+                er += self.scale_reads(q, 1 if p == 0 else 0)
+            e0, e1 = xs + 1, 5 * nm - 1
+            for n, r in enumerate(er):
+                post[e0 + n * (e1 - e0) // len(er)].append(r)
         # Y
-        if flavor == "steady":
-            wy = WaitVm(("X", -1), {"s": nx + 4})
-        elif flavor == "first0":
-            wy = WaitVm(("X", -1), {"a": nx + 4, "b": nx + 4 + NST, "c": nx})
-        elif flavor == "first0_fe":
-            wy = WaitVm(("X", -1), {"d": nx + 4 + sy})
-        else:   # first1: X of step 0 is awaited; a fused epilogue issued part of its stores behind that
-            wy = WaitVm(("X", -1), {"a": nx + 4 + nsc, "b": nx + 4 + nsc, "c": nx + 4 + nsc, "d": nx + 4 + nsc})
+        wy = WaitVm(("X", -1), keys)
         pre[tail0] += [Op("s_waitcnt lgkmcnt(0)"), wy, Op("s_barrier")]
         tail = total - tail0
-        q = p ^ 1
         if prefetch:
             lds = []
-            if self.fp4 and p == 1:
-                # the next step opens a new scale group: it sits in the other buffer
-                post[tail0] += [Op(f"v_xor_b32 v240, {SCBUF}, v240"), Op(f"v_xor_b32 v241, {SCBUF}, v241")]
-            for j in range(8):
-                lds += self.frag_read(self.vB(q, j), 1, q, j)
-            if self.fp4:
+            if not sc_early:
+                post[tail0] += sc_flip
+            for jb in range(4 if early else 0, 8):
+                lds += self.frag_read(self.vB(q, jb), 1, q, jb)
+            if self.fp4 and not sc_early:
                 lds += self.scale_reads(q, 1 if p == 0 else 0)
             lds += self.frag_read(self.vA(0), 0, q, 0)
             span = tail // 2
@@ -368,13 +377,67 @@ class Gen:
             a2 = max(tail0 + tail * 5 // 6, 7 * nm)
             post[a1] += self.frag_read(self.vA(1), 0, q, 1)
             post[a2] += self.frag_read(self.vA(2), 0, q, 2)
-        for n, op in enumerate(hi):
-            place(tail0 + n * (tail - 2) // len(hi), op)
+        for n, op in enumerate(a_hi):
+            place(tail0 + n * (tail - 2) // len(a_hi), op)
         post[total - 2] += adv_a
+        body = []
         for m in range(total):
-            out += pre[m]
-            out.append(self.mfma(p, m // nm, m % nm, first0))
-            out += post[m]
+            body += pre[m]
+            body.append(self.mfma(p, m // nm, m % nm, first0))
+            body += post[m]
+        return out + self.lgkm_pass(body, pending0 if pending0 is not None else self.pending_at_step_start(p))
+
+    # ---- LDS read completion -----------------------------------------------------------------------------
+    @staticmethod
+    def _vregs(tok):
+        m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.fullmatch(r"v(\d+)", tok)
+        return {int(m.group(1))} if m else set()
+
+    def pending_at_step_start(self, p):
+        """What a step may find in flight when it follows a step that prefetched for it: everything but
+        A fragments 1 and 2 is older than those four reads."""
+        older = set(range(self.vB(p, 0), self.vB(p, 0) + 64)) | set(range(self.vA(0), self.vA(0) + 8))
+        if self.fp4:
+            older |= set(range(self.scA(p, 0), self.scA(p, 0) + 16))
+        a1, a2 = self.vA(1), self.vA(2)
+        return [older, set(range(a1, a1 + 4)), set(range(a1 + 4, a1 + 8)), set(range(a2, a2 + 4)), set(range(a2 + 4, a2 + 8))]
+
+    @classmethod
+    def read_dests(cls, ops):
+        return [cls._vregs(o.text.split()[1].rstrip(",")) for o in ops if isinstance(o, Op) and o.text.startswith("ds_read")]
+
+    def lgkm_pass(self, ops, pending):
+        """LDS reads complete in issue order; s_waitcnt lgkmcnt(n) lets the n youngest stay in flight.  Walks
+        the instructions of a step and puts such a wait in front of every instruction that reads a register an
+        LDS read in flight is going to write (the explicit lgkmcnt(0) in front of the barriers stay: they keep
+        a wave from declaring LDS rows free that its own reads have not left yet)."""
+        pending = list(pending)
+        out = []
+        for o in ops:
+            if isinstance(o, WaitVm):
+                out.append(o)
+                continue
+            t = o.text
+            if t.startswith("ds_read"):
+                pending.append(self._vregs(t.split()[1].rstrip(",")))
+            elif t.startswith("s_waitcnt lgkmcnt("):
+                n = int(t[t.index("(") + 1:t.index(")")])
+                pending = pending[len(pending) - n:] if n else []
+            elif t.startswith("v_") or t.startswith("global_"):
+                # (every vector register the instruction names, its destination included: writing a register
+                # that an LDS read in flight is about to overwrite would be just as wrong)
+                srcs = set()
+                for x in t.split()[1:]:
+                    srcs |= self._vregs(x.rstrip(","))
+                hit = max((k for k, d in enumerate(pending) if d & srcs), default=-1)
+                if hit >= 0:
+                    n = min(15, len(pending) - 1 - hit)
+                    out.append(Op(f"s_waitcnt lgkmcnt({n})"))
+                    pending = pending[len(pending) - n:] if n else []
+            out.append(o)
         return out
 
     # ---- the whole K loop of one tile -------------------------------------------------------------------
@@ -383,9 +446,10 @@ class Gen:
         if self.fp4:
             for op in self.scale_dma(False, ("Y", -2)):
                 out += op
-        for st, tags in ((0, (("Y", -2), ("Y", -2), ("Y", -2))), (1, (("X", -1), ("X", -1), ("Y", -1)))):
+        xb = ("XB", -1) if self.earlyb else ("X", -1)
+        for st, tags in ((0, (("Y", -2), ("Y", -2), ("Y", -2), ("Y", -2))), (1, (xb, ("X", -1), ("X", -1), ("Y", -1)))):
             ops = self.dma(st, False, None)
-            for grp, idx in zip(tags, ((8, 9, 10, 11, 12, 13, 14, 15), (0, 1, 4, 5), (2, 3, 6, 7))):   # B, A lo, A hi: the order the steps use
+            for grp, idx in zip(tags, ((8, 9, 12, 13), (10, 11, 14, 15), (0, 1, 4, 5), (2, 3, 6, 7))):   # B lo, B hi, A lo, A hi: the order the steps use
                 for n in idx:
                     ops[n][-1].vm = grp
                     out += ops[n]
@@ -428,8 +492,9 @@ class Gen:
         # (either way s79 now names the buffer the NEXT scale group goes to)
         P["entry_fe"] = self.scale_reads_epi() if self.scaled_epi else []
         P["entry"] = [Op(f"s_mov_b32 s{S_AFTER}, 1")] + self.entry_reads()
-        P["first0"] = self.step(0, False, True, "first0")
-        P["first0_fe"] = self.step(0, False, True, "first0_fe")
+        # (step 0 of a tile follows the entry reads: exactly those may be in flight)
+        P["first0"] = self.step(0, False, True, "first0", self.read_dests(P["entry"]))
+        P["first0_fe"] = self.step(0, False, True, "first0_fe", self.read_dests(P["entry_fe"] + P["entry"]))
         P["first1"] = self.step(1, False, True, "first1")
         P["steady0"] = self.step(0, False, True)
         P["steady1"] = self.step(1, False, True)
@@ -446,6 +511,7 @@ class Gen:
             # the buffer that holds the next tile's first scale group
             end.append(Op(f"s_xor_b32 %[scbuf], s{S_SCN}, {SCBUF}"))
         P["end"] = end
+        self.solve(P)
         return P
 
     # ---- text ---------------------------------------------------------------------------------------------
@@ -524,16 +590,13 @@ class Gen:
     def text(self):
         return "".join(f'  "{l}\\n\\t"\n' for l in self.program())
 
-    # ---- checker ----------------------------------------------------------------------------------------------
-    def check(self):
+    # ---- wait counts: solved and checked by replay -----------------------------------------------------------
+    def replay(self, P, visit):
         """Replays the vector-memory operations of every history a tile can have (first tile of the
         workgroup; after a tile whose epilogue ran as compiled code with 32 stores, or with an unknown
         number -- tried with none and with many; after a tile whose epilogue is fused into this one) for
-        tiles of 4, 6 and 8 K steps, two tiles in a row, and checks at every wait that the number it
-        allows in flight does not exceed the number of operations issued after the awaited group."""
-        P = self.parts()
-        worst = {}
-
+        tiles of 4, 6, 8 and 10 K steps, three tiles in a row, and calls visit(wait, history key, number of
+        operations issued after the awaited group, where) at every wait."""
         def run(seq):
             """seq: list of (part name, step number, history key or None)"""
             q = []       # tags in issue order
@@ -546,32 +609,59 @@ class Gen:
                         grp = (o.awaits[0], o.awaits[1] + step)
                         key = hist if hist in o.vals else ("s" if "s" in o.vals else None)
                         assert key is not None, (name, step, hist, o.vals)
-                        n = o.vals[key]
                         idx = max((i for i, t in enumerate(q) if t == grp), default=-1)
                         assert idx >= 0, f"{self.kind}: {name} step {step} waits for {grp}, which nobody issued"
-                        allowed = len(q) - 1 - idx
-                        assert n <= allowed, f"{self.kind}: {name} step {step} history {hist}: waits vmcnt({n}) for {grp}, only {allowed} younger operations exist"
-                        worst[(name, o.awaits, key)] = min(worst.get((name, o.awaits, key), 99), allowed - n)
+                        visit(o, key, len(q) - 1 - idx, f"{self.kind}: {name} step {step} history {hist}: wait for {grp}")
                     elif o.vm is not None:
                         q.append((o.vm[0], o.vm[1] + step))
-            return q
 
-        def tile(base, ksteps, hist0, after_hist):
+        def tile(base, ksteps, hist0):
             """parts of one tile whose step 0 is number `base`"""
-            s = [("first0_fe" if hist0 == "d" else "first0", base, hist0), ("first1", base + 1, hist0)]
+            t = [("first0_fe" if hist0 == "d" else "first0", base, hist0), ("first1", base + 1, hist0)]
             h = "f"
             for it in range(2, ksteps - 2, 2):
-                s += [("steady0", base + it, h), ("steady1", base + it + 1, "s")]
+                t += [("steady0", base + it, h), ("steady1", base + it + 1, "s")]
                 h = "s"
-            s += [("last0", base + ksteps - 2, h), ("last1", base + ksteps - 1, "s")]
-            return s
+            t += [("last0", base + ksteps - 2, h), ("last1", base + ksteps - 1, "s")]
+            return t
 
-        for k in (4, 6, 8):
+        for k in (4, 6, 8, 10):
             for hist, nstores in (("b", NST), ("c", 0), ("c", 50), ("d", 0)):
-                seq = [("prologue", 0, "a")] + tile(0, k, "a", None)
-                seq += [("cstores", k, nstores)] + tile(k, k, hist, None)
-                seq += [("cstores", 2 * k, NST)] + tile(2 * k, k, "b", None)
+                seq = [("prologue", 0, "a")] + tile(0, k, "a")
+                seq += [("cstores", k, nstores)] + tile(k, k, hist)
+                seq += [("cstores", 2 * k, NST)] + tile(2 * k, k, "b")
                 run(seq)
+
+    def solve(self, P):
+        """vmcnt counts loads and stores in issue order: a wait for a group of copies may leave as many
+        operations in flight as were issued after that group -- in EVERY history that reaches the wait.
+        Fills in the counts that the steps left open with the smallest such number."""
+        found = {}
+
+        def visit(o, key, younger, where):
+            if o.vals[key] is None:
+                found[(id(o), key)] = min(found.get((id(o), key), 63), younger)
+        self.replay(P, visit)
+        for part in P.values():
+            for o in part:
+                if isinstance(o, WaitVm):
+                    for key in o.vals:
+                        if o.vals[key] is None:
+                            o.vals[key] = found.get((id(o), key), 0)    # (a history that never reaches the wait: drain)
+
+    def check(self):
+        """Replays every history (see replay) and checks at every wait that the number it allows in flight
+        does not exceed the number of operations issued after the awaited group.  Returns the slack per
+        wait site."""
+        P = self.parts()
+        worst = {}
+
+        def visit(o, key, younger, where):
+            n = o.vals[key]
+            assert n <= younger, f"{where}: vmcnt({n}), only {younger} younger operations exist"
+            site = (where.split(":")[1].split(" step")[0].strip(), o.awaits, key)
+            worst[site] = min(worst.get(site, 99), younger - n)
+        self.replay(P, visit)
         return worst
 
 

@@ -106,8 +106,11 @@ void read_hooks() {
   g_hooks.quant_div64 = env_int("TB_QUANT_DIV64", 0);
   g_hooks.lab = env_int("TB_DEBUG", 0);
 }
-const Hooks& hooks() {
+std::mutex g_hooks_mu;
+// (a copy taken under the hooks' own lock: tb_debug_option may change one while another thread plans)
+Hooks hooks() {
   std::call_once(g_hooks_once, read_hooks);
+  std::lock_guard<std::mutex> lk(g_hooks_mu);
   return g_hooks;
 }
 
@@ -466,27 +469,25 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream);
 // score tiles again (a persistent tb_gemm that considers a column split makes three plans and prices
 // two sub-problems).
 struct PlanKey {
-  int64_t v[30];
+  int64_t v[56];
   bool operator==(const PlanKey& o) const { return std::memcmp(v, o.v, sizeof(v)) == 0; }
 };
+// (every field in a slot of its own: packed fields of a descriptor with a negative or oversized value would
+// overlap and let one job find another job's plan, or its cached error)
 PlanKey plan_key(const Job& j, int dev) {
   PlanKey k;
   std::memset(&k, 0, sizeof(k));
   auto al = [](const void* q) { return (int64_t)((uintptr_t)q & 255) | (q ? 256 : 0); };
   int i = 0;
-  k.v[i++] = ((int64_t)j.dt) | ((int64_t)j.c_type << 8) | ((int64_t)j.bias_type << 16) | ((int64_t)j.schedule << 24) | ((int64_t)dev << 32);
-  k.v[i++] = j.M; k.v[i++] = j.N; k.v[i++] = j.K;
-  k.v[i++] = j.a_sr; k.v[i++] = j.a_sk; k.v[i++] = j.b_sr; k.v[i++] = j.b_sk; k.v[i++] = j.c_sm; k.v[i++] = j.c_sn;
-  k.v[i++] = j.mxa_sr; k.v[i++] = j.mxa_sk; k.v[i++] = j.mxb_sr; k.v[i++] = j.mxb_sk; k.v[i++] = j.bias_stride;
-  k.v[i++] = ((int64_t)j.bm) | ((int64_t)j.bn << 16) | ((int64_t)j.bk << 32) | ((int64_t)j.group_m << 48);
-  k.v[i++] = ((int64_t)j.num_xcds) | ((int64_t)j.grid << 16) | ((int64_t)j.counters_per_xcd << 48);
-  k.v[i++] = ((int64_t)j.ws_mode) | ((int64_t)j.ws_local << 8) | ((int64_t)j.cu_mask_len << 40);
-  k.v[i++] = j.ws_global;
-  k.v[i++] = ((int64_t)j.num_groups) | ((int64_t)j.grp_phase << 16) | ((int64_t)j.grp_big << 24) | ((int64_t)j.grp_thr << 40) | ((int64_t)j.grp_auto << 56);
-  k.v[i++] = j.b_group_stride; k.v[i++] = j.sb_group_stride;
-  k.v[i++] = al(j.A) | (al(j.B) << 10) | (al(j.C) << 20) | (al(j.mxa) << 30) | (al(j.mxb) << 40) | (al(j.bias) << 50);
-  k.v[i++] = (j.sa ? 1 : 0) | (j.sb ? 2 : 0) | (j.cu_mask ? 4 : 0) | (j.group_offsets ? 8 : 0) | ((int64_t)(j.column_split & 3) << 4);
-  k.v[i++] = (int64_t)g_hooks_version;
+  const int64_t f[] = {
+      j.dt, j.c_type, j.bias_type, j.schedule, dev, j.M, j.N, j.K, j.a_sr, j.a_sk, j.b_sr, j.b_sk, j.c_sm, j.c_sn,
+      j.mxa_sr, j.mxa_sk, j.mxb_sr, j.mxb_sk, j.bias_stride, j.bm, j.bn, j.bk, j.group_m, j.num_xcds, j.grid,
+      j.counters_per_xcd, j.ws_mode, j.ws_local, j.cu_mask_len, j.ws_global, j.num_groups, j.grp_phase, j.grp_big,
+      j.grp_thr, j.grp_auto, j.b_group_stride, j.sb_group_stride, al(j.A), al(j.B), al(j.C), al(j.mxa), al(j.mxb),
+      al(j.bias), j.sa ? 1 : 0, j.sb ? 1 : 0, j.cu_mask ? 1 : 0, j.group_offsets ? 1 : 0, j.column_split,
+      (int64_t)g_hooks_version};
+  static_assert(sizeof(f) <= sizeof(k.v), "PlanKey too small");
+  for (int64_t x : f) k.v[i++] = x;
   return k;
 }
 // the fields of a plan that name memory or change from call to call
@@ -741,6 +742,7 @@ int tb_debug_option(const char* name, int value) {
   if (!name) return TB_ERR_NULL_POINTER;
   (void)hooks();
   std::lock_guard<std::mutex> lk(g_plan_mu);
+  std::lock_guard<std::mutex> lk2(g_hooks_mu);
   struct { const char* n; int* p; } table[] = {
       {"waves", &g_hooks.waves}, {"no_mxlds", &g_hooks.no_mxlds}, {"no_cline", &g_hooks.no_cline},
       {"no_skinny", &g_hooks.no_skinny}, {"skinny", &g_hooks.skinny}, {"grid", &g_hooks.grid}, {"panel", &g_hooks.panel},
@@ -833,6 +835,25 @@ int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream) {
   // call records nothing that a replay of a captured graph would repeat wrongly.
   j.epoch = TB_EPOCH_ON_DEVICE;
   return launch_columns(j, (hipStream_t)stream);
+}
+
+int tb_static_workspace_status(int* status, int clear) {
+  if (!status) return TB_ERR_NULL_POINTER;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return TB_ERR_NO_DEVICE;
+  std::call_once(g_scratch_once[dev], init_scratch, dev);
+  ScratchState& sc = g_scratch[dev];
+  if (sc.status != TB_OK) return sc.status;
+  // (the status word is control word CTL_STATUS of the array; the copy waits for the device's earlier work)
+  uint32_t word = 0;
+  uint8_t* at = (uint8_t*)sc.ptr + CTL_STATUS * 4;
+  if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(&word, at, 4, hipMemcpyDeviceToHost) != hipSuccess) return TB_ERR_LAUNCH;
+  if (clear && word != 0) {
+    const uint32_t zero = 0;
+    if (hipMemcpy(at, &zero, 4, hipMemcpyHostToDevice) != hipSuccess) return TB_ERR_LAUNCH;
+  }
+  *status = (int)word;
+  return TB_OK;
 }
 
 size_t tb_workspace_bytes(const tb_gemm_desc* desc) {

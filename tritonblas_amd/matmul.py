@@ -18,7 +18,8 @@ _SELECTOR_CACHE = {}
 _SELECTOR_CACHE_MAX = 4096
 # Launch state for entry points that are called without a MatmulConfig (tb.matmul(..., enable_streamk=True)
 # and friends): one workspace per (device, stream), grown on demand.  Epoch tags make zeroing between
-# launches unnecessary, and launches on one stream are ordered, so they can share it.
+# launches unnecessary, and launches on one stream are ordered, so they can share it.  Entries are never
+# dropped: a launch captured into a HIP graph keeps the raw pointer of the workspace it was given.
 _STREAM_CONFIGS = {}
 
 
@@ -26,8 +27,6 @@ def _stream_config(dev) -> MatmulConfig:
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
     cfg = _STREAM_CONFIGS.get(key)
     if cfg is None:
-        if len(_STREAM_CONFIGS) >= 64:
-            _STREAM_CONFIGS.clear()
         cfg = MatmulConfig(device=dev, workspace=None)
         _STREAM_CONFIGS[key] = cfg
     return cfg

@@ -60,7 +60,9 @@ def _quant(x: torch.Tensor, hadamard: bool, out=None):
     if not x.is_cuda:
         raise RuntimeError("tritonblas_amd: the MXFP4 quantiser runs on the GPU only")
     if x.stride(1) != 1 or x.data_ptr() % 16 or (x.stride(0) * x.element_size()) % 16:
-        x = x.contiguous()      # (the kernel reads rows with 16-byte loads)
+        # the kernel reads rows with 16-byte loads (a contiguous view that merely starts off a 16-byte
+        # boundary needs a real copy: .contiguous() would hand the same memory back)
+        x = x.clone(memory_format=torch.contiguous_format)
     if out is None:
         codes = torch.empty((M, N // 2), dtype=torch.uint8, device=x.device)
         scales = torch.empty((M, N // 32), dtype=torch.uint8, device=x.device)
