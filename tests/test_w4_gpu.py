@@ -109,14 +109,19 @@ def _fp4_case(m, n, k, seed):
     return torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs), torch.from_numpy(ws)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 256, 1024), (256, 256, 4096), (512, 768, 1024), (300, 500, 1536), (2048, 1280, 2048)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 1024), (256, 256, 4096), (512, 768, 1024), (300, 500, 1536), (2048, 1280, 2048),
+                                   (300, 500, 3072), (768, 512, 5120)])
 def test_fp4_four_wave_kernel(m, n, k, tb_option):
+    """The 4-wave MXFP4 kernel against the oracle and, bit for bit, against the 8-wave kernel."""
     import tritonblas_amd as tb
     _say(f"w4 fp4 {m}x{n}x{k}")
     xq, wq, xs, ws = _fp4_case(m, n, k, 75)
-    # scale bytes far from 127 in some blocks: the E8M0 operands of the scaled MFMA must be honoured
+    # scale bytes far from 127 in some blocks, different in every K block of a row: the E8M0 operands of the scaled
+    # MFMA must be honoured, and a scale byte that ends up with the wrong K block must show
     xs[::3, ::2] = 120
     ws[1::4, 1::3] = 133
+    xs[5::7, :] = (118 + torch.arange(k // 32) % 19).to(torch.uint8)
+    ws[2::5, :] = (136 - torch.arange(k // 32) % 17).to(torch.uint8)
     outs = {}
     for waves in (22, 24):
         tb_option("waves", waves)
@@ -205,7 +210,7 @@ def _launcher(kind, m, n, k, seed):
 
 @pytest.mark.parametrize("kind,bk", [("fp8", 128), ("fp4", 256), ("bf16", 64), ("i8", 128)])
 @pytest.mark.parametrize("m,n,steps,grid", [(512, 768, 4, 1), (512, 768, 6, 2), (300, 500, 8, 1), (1280, 768, 10, 3), (1100, 1300, 4, 2),
-                                            (4096, 8192, 4, 0)])
+                                            (4096, 8192, 4, 0), (768, 1100, 12, 2), (1280, 768, 16, 3), (4096, 4096, 8, 0)])
 def test_fused_epilogue(kind, bk, m, n, steps, grid, tb_option):
     """A workgroup that runs several tiles stores a full bf16 tile from inside the next tile's first K
     step.  With 1 to 3 workgroups for 6 to 30 tiles (and 512 tiles on the whole chip), whole and ragged

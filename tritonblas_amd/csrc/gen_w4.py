@@ -329,7 +329,7 @@ class Gen:
         def place(slot, op):
             """A copy needs one wait state between the write of m0 and its use: the MFMA of the slot is
             that instruction (m0 setup in front of it, the copy right behind)."""
-            if len(op) == 3 and not ({"nodma", "dmaonce", "m0nop"} & self.lab):
+            if len(op) == 3 and op[1].text == "s_nop 0" and not ({"nodma", "dmaonce", "m0nop"} & self.lab):
                 assert slot not in m0_slots
                 m0_slots.add(slot)
                 pre[slot].append(op[0])
