@@ -49,6 +49,23 @@ def timed(fn, steps, warmup, settle_ms=0.0):
     return start.elapsed_time(end) / steps, wall_ms
 
 
+def timed_rotating(fns, steps, warmup):
+    """HBM-bound kernels on cold data: back-to-back launches that cycle through several operand sets which together
+    exceed the 256 MB memory-side cache (what one launch leaves there is gone when its set comes up again), with no
+    flush in between whose write-back would share the memory bus with the timed kernel.  Returns ms per launch."""
+    n = len(fns)
+    for i in range(warmup):
+        fns[i % n]()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fns[i % n]()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
 def library_id():
     """First 12 hex digits of the SHA-256 of the shared library that is loaded: names the build a
     profile summary was taken from."""
@@ -217,11 +234,25 @@ def main():
         # fraction of the HBM peak is the flushed figure, the back-to-back one is cache assisted
         qms_cold = tb.do_bench(lambda: U.hadamard_mxfp4_quant(a4, out=qout), n_warmup=5, n_repeat=40, return_mode="median")
         qbytes = M4 * K4 * 2 + M4 * K4 // 2 + M4 * K4 // 32
-        sec["hadamard_mxfp4_quant_8192x16384"] = {"ms": round(qms_cold, 4), "GB/s": round(qbytes / qms_cold / 1e6, 1),
-                                                  "frac_hbm_peak": round(qbytes / qms_cold / 1e6 / PEAK_HBM_GBPS, 4),
-                                                  "timing": "median of 40 launches, caches flushed before each",
+        # third way, and the one the HBM fraction is taken from: four operand sets in turn (4 x 340 MB against a 256 MB
+        # memory-side cache), back to back, nothing flushed; a plain device copy that moves as many bytes, timed the
+        # same way over four buffer pairs, is the yard-stick
+        xsets = [a4] + [a4.roll(i + 1, 0) for i in range(3)]
+        osets = [qout] + [(torch.empty_like(qout[0]), torch.empty_like(qout[1])) for _ in range(3)]
+        qms_rot = timed_rotating([(lambda x=x, o=o: U.hadamard_mxfp4_quant(x, out=o)) for x, o in zip(xsets, osets)], steps2 * 4, 8)
+        csrc = [torch.empty(qbytes // 2, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
+        cdst = [torch.empty_like(x) for x in csrc]
+        copy_rot = timed_rotating([(lambda x=x, y=y: y.copy_(x)) for x, y in zip(csrc, cdst)], steps2 * 4, 8)
+        del xsets, osets, csrc, cdst
+        sec["hadamard_mxfp4_quant_8192x16384"] = {"ms": round(qms_rot, 4), "GB/s": round(qbytes / qms_rot / 1e6, 1),
+                                                  "frac_hbm_peak": round(qbytes / qms_rot / 1e6 / PEAK_HBM_GBPS, 4),
+                                                  "timing": "four operand sets in turn (1.36 GB > the 256 MB memory-side cache), back to back, no flush",
+                                                  "plain_copy_of_as_many_bytes_same_way_ms": round(copy_rot, 4),
+                                                  "plain_copy_GB/s": round(qbytes / copy_rot / 1e6, 1),
+                                                  "flushed_ms": round(qms_cold, 4), "flushed_GB/s": round(qbytes / qms_cold / 1e6, 1),
                                                   "hot_ms": round(qms, 4), "hot_GB/s": round(qbytes / qms / 1e6, 1),
-                                                  "note": "bf16 in, codes + E8M0 scales out, outputs preallocated"}
+                                                  "note": "bf16 in, codes + E8M0 scales out, outputs preallocated; flushed = the "
+                                                          "reference's do_bench loop (512 MiB rewritten before every launch), hot = one set back to back"}
         aq4, as4 = qout
         bq4, bs4 = U.hadamard_mxfp4_quant(b4)
         a4_sample = a4[:128].float().cpu().numpy()
@@ -229,8 +260,31 @@ def main():
         c4 = torch.empty(M4, N4, dtype=torch.bfloat16, device=dev)
         fms, _ = timed(lambda: tb.matmul_fp4(aq4, bq4, c4, as4, bs4), steps2, warm2, settle_ms=40.0)
         tf4 = 2.0 * M4 * N4 * K4 / fms / 1e9
-        sec["mxfp4_gemm_8192x8192x16384"] = {"ms": round(fms, 4), "TFLOP/s": round(tf4, 1),
-                                             "frac_mfma_peak": round(tf4 / PEAK_TFLOPS["mxfp4"], 4)}
+        clock4 = profile_summary("mxfp4_gemm_8192x8192x16384_mfma_busy")
+        sec["mxfp4_gemm_8192x8192x16384"] = {
+            "ms": round(fms, 4), "TFLOP/s": round(tf4, 1), "frac_mfma_peak": round(tf4 / PEAK_TFLOPS["mxfp4"], 4),
+            "roofline": {"bound": "mfma", "achieved": round(tf4, 1), "peak": PEAK_TFLOPS["mxfp4"], "unit": "TFLOP/s",
+                         "frac": round(tf4 / PEAK_TFLOPS["mxfp4"], 4),
+                         "sustained_clock_ghz": clock4["engine_clock_ghz"] if clock4 else None,
+                         "mfma_busy_in_cycles": clock4["mfma_busy"] if clock4 else None,
+                         "counters_from": f"profiles/mxfp4_gemm_8192x8192x16384_mfma_busy.json, library {clock4['library_id']}" if clock4
+                                          else "no counter summary of this library build is committed"}}
+        # parity spot check and CPU baseline: the oracle's GEMM of the dequantised operands on rows spread over the output
+        rows4 = torch.arange(0, M4, 4)[:2048] if not args.skip_cpu else torch.arange(0, M4, 613)[:14]
+        a_rows, as_rows, b_cpu4, bs_cpu4 = aq4[rows4].cpu(), as4[rows4].cpu(), bq4.cpu(), bs4.cpu()
+        best4, want4 = None, None
+        for _ in range(1 if args.skip_cpu else 2):
+            t0 = time.perf_counter()
+            want4 = OG.ref_gemm_fp4(a_rows, b_cpu4, as_rows, bs_cpu4, return_fp32=True)
+            dt = time.perf_counter() - t0
+            best4 = dt if best4 is None else min(best4, dt)
+        sec["mxfp4_gemm_8192x8192x16384"]["parity_rel_fro"] = float(f"{OG.rel_fro_error(c4[rows4].float().cpu(), want4.to(torch.bfloat16).float()):.3e}")
+        if not args.skip_cpu:
+            sec["mxfp4_gemm_8192x8192x16384"]["cpu_baseline"] = {
+                "value": round(2.0 * len(rows4) * N4 * K4 / best4 / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"every fourth row, {len(rows4)} rows, of the same GEMM ({len(rows4)}x{N4}x{K4}): oracle dequantisation (numpy) of both "
+                          f"operands + fp32 torch.mm, best of 2, {best4:.2f} s"}
+        del a_rows, as_rows, b_cpu4, bs_cpu4, want4
         q_sample = (aq4[:128].cpu().numpy(), as4[:128].cpu().numpy())
         del aq4, bq4, c4
         # fp16 1024^3 (the plumbing configuration): launch bound, so the host's share of a call matters
@@ -275,10 +329,21 @@ def main():
         dms, _ = timed(decode, steps2 * 4, warm2)
         dms_cold = tb.do_bench(decode, n_warmup=5, n_repeat=40, return_mode="median")
         dbytes = Md * Kd + Nd * Kd + Md * Nd * 2 + (Md + Nd) * 4
-        sec["fp8_decode_32x8192x28672"] = {"ms": round(dms_cold, 4), "GB/s": round(dbytes / dms_cold / 1e6, 1),
-                                           "frac_hbm_peak": round(dbytes / dms_cold / 1e6 / PEAK_HBM_GBPS, 4),
-                                           "timing": "median of 40 launches, caches flushed before each (the 235 MB weight "
-                                                     "otherwise stays in the 256 MB memory-side cache)",
+        # cold data without a flush: four weight matrices in turn (4 x 235 MB against the 256 MB memory-side cache);
+        # yard-stick: a plain device copy that moves as many bytes, four buffer pairs in turn
+        wsets = [wqd] + [wqd.roll(i + 1, 0) for i in range(3)]
+        dms_rot = timed_rotating([(lambda w=w: tb.matmul_a8w8_lt(aqd, w.T, sad, swd, cd, seld, cfgd, enable_streamk=True)) for w in wsets],
+                                 steps2 * 4, 8)
+        csrc = [torch.empty(dbytes // 2, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
+        cdst = [torch.empty_like(x) for x in csrc]
+        dcopy_rot = timed_rotating([(lambda x=x, y=y: y.copy_(x)) for x, y in zip(csrc, cdst)], steps2 * 4, 8)
+        del wsets, csrc, cdst
+        sec["fp8_decode_32x8192x28672"] = {"ms": round(dms_rot, 4), "GB/s": round(dbytes / dms_rot / 1e6, 1),
+                                           "frac_hbm_peak": round(dbytes / dms_rot / 1e6 / PEAK_HBM_GBPS, 4),
+                                           "timing": "four weight matrices in turn (940 MB > the 256 MB memory-side cache), back to back, no flush",
+                                           "plain_copy_of_as_many_bytes_same_way_ms": round(dcopy_rot, 4),
+                                           "plain_copy_GB/s": round(dbytes / dcopy_rot / 1e6, 1),
+                                           "flushed_ms": round(dms_cold, 4), "flushed_GB/s": round(dbytes / dms_cold / 1e6, 1),
                                            "hot_ms": round(dms, 4), "hot_GB/s": round(dbytes / dms / 1e6, 1),
                                            "host_us_per_call": round(host_us_per_call(decode), 2),
                                            "kernel": f"enable_streamk=True call; the library picks between the Stream-K tile kernel "

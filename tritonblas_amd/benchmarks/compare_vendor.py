@@ -1,7 +1,7 @@
 """Side-by-side timing of this library and the vendor library PyTorch dispatches to (hipBLASLt through
 torch.matmul / torch._scaled_mm) on the same tensors.
 
-    python -m tritonblas_amd.benchmarks.compare_vendor [--shapes fp8,bf16,decode] [--steps 40] [--settle-ms 40]
+    python -m tritonblas_amd.benchmarks.compare_vendor [--shapes fp8,bf16,decode,mxfp4] [--steps 40] [--settle-ms 40]
 
 Cases: "fp8" = a8w8 8192x28672x8192 with per-row / per-column scales (torch._scaled_mm row-wise is the
 same operation; its tensor-wise form, one scale per tensor, is the simpler problem the vendor ships a
@@ -9,7 +9,10 @@ hand-written kernel for) and "bf16" = 8192^3 with K-major operands.  Every timin
 `settle-ms` of untimed launches of the same call (the engine clock needs tens of milliseconds of load
 to settle) and is the average of `steps` back-to-back launches between two events.  "decode" = a8w8
 32x8192x28672 (the 235 MB weight is the traffic): timed back to back and with the caches flushed before
-every launch (do_bench), next to a plain device copy of as many bytes under the same flush.  One JSON line per
+every launch (do_bench), next to a plain device copy of as many bytes under the same flush.  "mxfp4" = the MXFP4
+GEMM 8192x8192x16384 (e2m1 codes, one E8M0 scale per 32 values of K) against torch._scaled_mm on the same packed
+operands and scale bytes (hipBLASLt's block-scaled kernel), with N(0,1) data and with all-zero codes (the second
+shows what the kernels do when the engine clock is not held down by the power of the multipliers).  One JSON line per
 case on stdout.  Run it under `rocprofv3 --kernel-trace --stats` or `--pmc` to see the kernels behind
 each call.
 """
@@ -119,6 +122,39 @@ def case_decode(steps, settle_ms, dev):
     return out
 
 
+def case_mxfp4(steps, settle_ms, dev):
+    import tritonblas_amd as tb
+    import tritonblas_amd.utils as U
+    m, n, k = 8192, 8192, 16384
+    g = torch.Generator(device=dev).manual_seed(5)
+    a = torch.randn(m, k, device=dev, generator=g).bfloat16()
+    w = torch.randn(n, k, device=dev, generator=g).bfloat16()
+    aq, sa = U.dynamic_mxfp4_quant(a)
+    wq, sw = U.dynamic_mxfp4_quant(w)
+    del a, w
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    out = {"case": "mxfp4 8192x8192x16384, bf16 out", "flops": 2.0 * m * n * k}
+    out["this_library_ms"] = timed(lambda: tb.matmul_fp4(aq, wq, c, sa, sw), steps, settle_ms)
+    az, wz = torch.zeros_like(aq), torch.zeros_like(wq)
+    s1a, s1w = torch.full_like(sa, 127), torch.full_like(sw, 127)
+    out["this_library_zero_data_ms"] = timed(lambda: tb.matmul_fp4(az, wz, c, s1a, s1w), steps, settle_ms)
+    try:
+        f4, e8 = torch.float4_e2m1fn_x2, torch.float8_e8m0fnu
+        va, vw, vsa, vsw = aq.view(f4), wq.view(f4), sa.view(e8), sw.view(e8)
+        vendor = lambda x, y, p, q: torch._scaled_mm(x, y.t(), scale_a=p, scale_b=q, out_dtype=torch.bfloat16)
+        ref = vendor(va, vw, vsa, vsw)
+        tb.matmul_fp4(aq, wq, c, sa, sw)
+        torch.cuda.synchronize()
+        rows = slice(0, 512)
+        out["rel_fro_between_the_two"] = float(((c[rows].float() - ref[rows].float()).norm() / ref[rows].float().norm()).item())
+        del ref
+        out["vendor_ms"] = timed(lambda: vendor(va, vw, vsa, vsw), steps, settle_ms)
+        out["vendor_zero_data_ms"] = timed(lambda: vendor(az.view(f4), wz.view(f4), s1a.view(e8), s1w.view(e8)), steps, settle_ms)
+    except Exception as e:   # (block-scaled FP4 through torch is not there in every PyTorch / hipBLASLt build)
+        out["vendor_error"] = f"{type(e).__name__}: {str(e)[:200]}"
+    return out
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="fp8,bf16")
@@ -127,7 +163,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     dev = torch.device("cuda", torch.cuda.current_device())
     for name in args.shapes.split(","):
-        fn = {"fp8": case_fp8, "bf16": case_bf16, "decode": case_decode}.get(name.strip())
+        fn = {"fp8": case_fp8, "bf16": case_bf16, "decode": case_decode, "mxfp4": case_mxfp4}.get(name.strip())
         if fn is None:
             print(f"unknown case {name!r}", file=sys.stderr)
             return 2
