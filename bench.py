@@ -331,7 +331,7 @@ def main():
         dbytes = Md * Kd + Nd * Kd + Md * Nd * 2 + (Md + Nd) * 4
         # cold data without a flush: four weight matrices in turn (4 x 235 MB against the 256 MB memory-side cache);
         # yard-stick: a plain device copy that moves as many bytes, four buffer pairs in turn
-        wsets = [wqd] + [wqd.roll(i + 1, 0) for i in range(3)]
+        wsets = [wqd] + [wqd.view(torch.uint8).roll(i + 1, 0).view(wqd.dtype) for i in range(3)]
         dms_rot = timed_rotating([(lambda w=w: tb.matmul_a8w8_lt(aqd, w.T, sad, swd, cd, seld, cfgd, enable_streamk=True)) for w in wsets],
                                  steps2 * 4, 8)
         csrc = [torch.empty(dbytes // 2, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]

@@ -1184,9 +1184,6 @@ struct Sched {
     G = gridDim.x;
     gphase = p.mode == MODE_GROUPED ? grouped_phase(p, G) : 0;
     pid = blockIdx.x;
-#ifdef W4_LAB_XCDSWAP
-    pid ^= W4_LAB_XCDSWAP;   // measurement build: XCD x runs the tiles XCD x ^ W4_LAB_XCDSWAP would run
-#endif
     sk_id = blockIdx.x;
     if (p.mode != MODE_WS && p.num_xcds > 1) pid = chiplet_transform_chunked(pid, G, p.num_xcds, p.chunk);
     next_tile = pid;
