@@ -55,7 +55,9 @@ enum {
 enum {
   TB_SCHED_PERSISTENT = 0,    /* data parallel, resident grid loops over tiles (matmul.py:160-198)  */
   TB_SCHED_WORK_STEALING = 1, /* atomic tile queues per XCD x slot       (matmul.py:112-159)        */
-  TB_SCHED_STREAMK = 2        /* data parallel tiles + Stream-K tail     (matmul.py:202-366)        */
+  TB_SCHED_STREAMK = 2,       /* data parallel tiles + Stream-K tail     (matmul.py:202-366)        */
+  TB_SCHED_STREAMK_WS = 3     /* the same with the data parallel tiles drawn from the work-stealing queues
+                                 (matmul.py:279-323, kernels/streamk_gemm_work_stealing.py:9-418)   */
 };
 
 /* How work-stealing workgroups find tiles (kernels/persistent_gemm_work_stealing.py). */
@@ -186,6 +188,16 @@ size_t tb_workspace_bytes(const tb_gemm_desc* desc);
 #define TB_STATIC_WORKSPACE_BYTES (16u << 20)
 #define TB_EPOCH_ON_DEVICE 0xFFFFFFFFu
 int tb_gemm_static_workspace(const tb_gemm_desc* desc, void* stream);
+
+/* What a tb_gemm call with this descriptor would launch (nothing is launched): the tile, the kernel family
+ * (waves per workgroup; four_wave: the hand-scheduled 256x256 kernel), the grid, how many tiles form the Stream-K
+ * tail and in units of how many K steps their ranges are cut, whether the whole tiles come from the work-stealing
+ * queues, whether the small-M streaming kernel runs instead of a tile kernel.  For tests and for callers that log
+ * their launches; no counterpart in the reference (its launchers print the same facts when asked to be verbose). */
+typedef struct tb_launch_info {
+  int32_t block_m, block_n, block_k, waves, four_wave, mode, grid, total_tiles, sk_tiles, sk_unit, sk_ws, skinny;
+} tb_launch_info;
+int tb_gemm_launch_info(const tb_gemm_desc* desc, tb_launch_info* out);
 
 /* Reads the status word of the current GPU's static workspace into *status (1: a Stream-K launch through
  * tb_gemm_static_workspace ran into spin_limit and stored NaN tiles) and, with clear != 0, sets it back to 0.

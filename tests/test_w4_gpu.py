@@ -418,3 +418,101 @@ def test_a8w8_fp8_output(m, n, k, streamk):
     # the rounding itself: at most one e4m3 step away from the oracle's cast, and mostly identical
     same = (c.cpu().view(torch.uint8) == want.view(torch.uint8)).float().mean().item()
     assert same >= 0.99, f"only {same:.4f} of the e4m3 codes match the oracle's"
+
+
+# ---- Stream-K on the 4-wave kernels, and Stream-K with work stealing ------------------------------------------
+def _launch_info(a, b, c, schedule, grid, tile, scales=False):
+    from tritonblas_amd import _lib
+    import ctypes as C
+    d = _lib.tb_gemm_desc()
+    d.struct_bytes = C.sizeof(_lib.tb_gemm_desc)
+    d.a_type = d.b_type = _lib.tb_dtype(a.dtype)
+    d.c_type = _lib.tb_dtype(c.dtype)
+    d.m, d.k = a.shape
+    d.n = b.shape[1]
+    d.a_stride_m, d.a_stride_k = a.stride()
+    d.b_stride_k, d.b_stride_n = b.stride()
+    d.c_stride_m, d.c_stride_n = c.stride()
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.block_m, d.block_n, d.block_k = tile
+    d.schedule, d.grid = schedule, grid
+    info = _lib.tb_launch_info()
+    assert _lib.load().tb_gemm_launch_info(d, C.byref(info)) == _lib.TB_OK
+    return info
+
+
+@pytest.mark.parametrize("kind,bk", [("fp8", 128), ("bf16", 64)])
+@pytest.mark.parametrize("m,n,steps,grid", [(512, 512, 16, 12), (768, 512, 32, 7), (300, 500, 8, 5), (512, 768, 20, 9),
+                                            (1024, 1024, 64, 256), (2304, 2048, 8, 64)])
+@pytest.mark.parametrize("work_stealing", [False, True])
+def test_four_wave_streamk(kind, bk, m, n, steps, grid, work_stealing, tb_option):
+    """The Stream-K tail on the hand-scheduled kernels (K ranges cut at multiples of four K steps): oracle parity,
+    the same bits in three launches on one config without reset, the launch really is the 4-wave kernel, and with
+    the whole tiles drawn from the work-stealing queues the bits stay the same."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    k = steps * bk
+    _say(f"w4 stream-k {kind} {m}x{n}x{k} grid {grid} ws {work_stealing}")
+    if kind == "fp8":
+        aq, bq, sa, sb = _fp8_case(m, n, k, 84)
+        a, b = aq.cuda(), bq.T.contiguous().cuda().T
+        scales = dict(a_scale=sa.cuda(), b_scale=sb.cuda(), quantized=True)
+        want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).to(torch.bfloat16)
+        tol = TOL_Q
+    else:
+        g = torch.Generator().manual_seed(84)
+        a_cpu = (torch.randn(m, k, generator=g) * 0.5).bfloat16()
+        bt_cpu = (torch.randn(n, k, generator=g) * 0.5).bfloat16()
+        a, b = a_cpu.cuda(), bt_cpu.cuda().T
+        scales = {}
+        want = OG.ref_gemm(a_cpu, bt_cpu.T, torch.float32).to(torch.bfloat16)
+        tol = 1e-3
+    tb_option("waves", 22)
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.bfloat16, a.device, streamk=True)
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, bk
+    c = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    sched = _lib.TB_SCHED_STREAMK_WS if work_stealing else _lib.TB_SCHED_STREAMK
+    info = _launch_info(a, b, c, sched, grid, (256, 256, bk))
+    tiles = ((m + 255) // 256) * ((n + 255) // 256)
+    if tiles % min(grid, 256) != 0:
+        assert info.four_wave == 1 and info.sk_unit == 4 and info.sk_tiles == tiles % info.grid
+        assert info.sk_ws == (1 if work_stealing else 0)
+    cfg = tb.matmul_preamble(sel)
+    outs = []
+    for rep in range(3):
+        c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=grid, work_stealing=work_stealing, **scales)
+        outs.append(c.cpu())
+    cfg.check()
+    assert OG.rel_fro_error(outs[0].float(), want.float()) <= tol
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    if work_stealing:
+        cs = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        streamk_matmul_lt(a, b, cs, sel, cfg, sk_grid=grid, **scales)
+        assert torch.equal(outs[0].view(torch.int16), cs.cpu().view(torch.int16)), "queues and static deal must give the same bits"
+
+
+def test_streamk_work_stealing_eight_wave_kernel(tb_option):
+    """The same schedule on a compiler-scheduled tile (128x128): whole tiles from the queues, Stream-K tail, same
+    bits as the static deal, three launches without reset."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import streamk_matmul_lt
+    m, n, k = 1536, 1280, 2048
+    g = torch.Generator().manual_seed(86)
+    a_cpu = (torch.randn(m, k, generator=g) * 0.5).bfloat16()
+    b_cpu = (torch.randn(k, n, generator=g) * 0.5).bfloat16()
+    want = OG.ref_gemm(a_cpu, b_cpu, torch.float32).to(torch.bfloat16)
+    a, b = a_cpu.cuda(), b_cpu.cuda()
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.bfloat16, a.device, streamk=True)
+    sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 128, 128, 64
+    cfg = tb.matmul_preamble(sel)
+    static = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    streamk_matmul_lt(a, b, static, sel, cfg, sk_grid=50)
+    assert OG.rel_fro_error(static.float().cpu(), want.float()) <= 1e-3
+    for rep in range(3):
+        c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        streamk_matmul_lt(a, b, c, sel, cfg, sk_grid=50, work_stealing=True)
+        assert torch.equal(c.view(torch.int16), static.view(torch.int16)), f"launch {rep}"
+    cfg.check()

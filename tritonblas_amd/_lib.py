@@ -20,14 +20,14 @@ TB_EPOCH_ON_DEVICE = 0xFFFFFFFF   # tb_gemm_desc.epoch: the workspace counts its
 TB_ERR_NULL_POINTER, TB_ERR_BAD_SHAPE, TB_ERR_BAD_DTYPE, TB_ERR_BAD_LAYOUT, TB_ERR_BAD_TILE = -1, -2, -3, -4, -5
 TB_ERR_WORKSPACE, TB_ERR_BAD_SCHEDULE, TB_ERR_LAUNCH, TB_ERR_NO_DEVICE, TB_ERR_BAD_ARGUMENT = -6, -7, -8, -9, -10
 TB_F16, TB_BF16, TB_FP8_E4M3, TB_FP4_E2M1, TB_F32, TB_I8, TB_FP8_E5M2 = 0, 1, 2, 3, 4, 5, 6
-TB_SCHED_PERSISTENT, TB_SCHED_WORK_STEALING, TB_SCHED_STREAMK = 0, 1, 2
+TB_SCHED_PERSISTENT, TB_SCHED_WORK_STEALING, TB_SCHED_STREAMK, TB_SCHED_STREAMK_WS = 0, 1, 2, 3
 TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
 
 EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
     "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
     "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile", "tb_hierarchical_split",
-    "tb_workspace_layout", "tb_debug_option", "tb_gemm_static_workspace", "tb_static_workspace_status",
+    "tb_workspace_layout", "tb_debug_option", "tb_gemm_static_workspace", "tb_static_workspace_status", "tb_gemm_launch_info",
 ]
 
 
@@ -35,6 +35,11 @@ class tb_hw(C.Structure):
     _fields_ = [("n_cu", C.c_int32), ("num_xcd", C.c_int32), ("cu_per_xcd", C.c_int32), ("lds_bytes", C.c_int32),
                 ("l2_bytes", C.c_int32), ("clock_khz", C.c_int32), ("mem_clock_khz", C.c_int32),
                 ("wave_size", C.c_int32), ("hbm_gbps", C.c_double), ("arch", C.c_char * 32)]
+
+
+class tb_launch_info(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("block_m", "block_n", "block_k", "waves", "four_wave", "mode", "grid", "total_tiles",
+                                         "sk_tiles", "sk_unit", "sk_ws", "skinny")]
 
 
 class tb_problem(C.Structure):
@@ -123,6 +128,7 @@ def load():
     lib.tb_ws_queue_tile.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32)] * 2
     lib.tb_hierarchical_split.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.tb_gemm_static_workspace.argtypes = [C.POINTER(tb_gemm_desc), C.c_void_p]
+    lib.tb_gemm_launch_info.argtypes = [C.POINTER(tb_gemm_desc), C.POINTER(tb_launch_info)]
     lib.tb_static_workspace_status.argtypes = [C.POINTER(C.c_int), C.c_int]
     lib.tb_static_workspace_status.restype = C.c_int
     lib.tb_workspace_layout.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]

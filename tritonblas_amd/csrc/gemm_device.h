@@ -68,6 +68,9 @@ struct GemmParams {
   int32_t debug;                 // measurement builds only (TB_LAB_HOOKS): bit0 skip global->LDS copies, bit1 skip MFMA work
   // Stream-K
   int32_t sk_tiles;
+  int32_t sk_unit;               // K steps per unit of the Stream-K split (0 or 1: single steps; the 4-wave kernels run K in
+                                 // blocks of four steps, so their ranges are cut at multiples of four)
+  int32_t sk_ws;                 // 1: the whole tiles in front of the Stream-K tail are drawn from the work-stealing queues
   float* P;
   uint32_t* flags;
   uint32_t epoch, spin_limit;
@@ -1179,6 +1182,7 @@ struct Sched {
   int64_t start, last, q, rem;  // Stream-K iteration range of this workgroup
   int dp_tiles;
   int gphase;             // grouped: which tile table this launch runs
+  bool ws_phase;          // Stream-K with work stealing: still drawing whole tiles from the queues
 
   __device__ __forceinline__ void init(const GemmParams& p) {
     G = gridDim.x;
@@ -1190,17 +1194,60 @@ struct Sched {
     step = 0;
     dp_tiles = p.total_tiles - p.sk_tiles;
     start = last = q = rem = 0;
+    ws_phase = false;
+    if constexpr (SK) ws_phase = p.mode == MODE_SK && p.sk_ws != 0;
     if (p.mode == MODE_SK) {
-      const int64_t total_sk = (int64_t)p.sk_tiles * p.k_iters;
+      const int64_t total_sk = (int64_t)p.sk_tiles * (p.k_iters / max(1, p.sk_unit));
       q = total_sk / G; rem = total_sk % G;
       // The iteration ranges follow the order in which the hardware starts workgroups (the raw id, not
       // the XCD-remapped one): a tile is finished by the workgroup that holds its LAST iterations, so
       // every wait is for a workgroup with a lower id, which has been started already -- the exchange
       // does not need the whole grid to be resident.
-      start = (int64_t)dp_tiles * p.k_iters + sk_id * q + min((int64_t)sk_id, rem);
-      last = (int64_t)dp_tiles * p.k_iters + (sk_id + 1) * q + min((int64_t)sk_id + 1, rem);
+      const int64_t ipt = p.k_iters / max(1, p.sk_unit);
+      start = (int64_t)dp_tiles * ipt + sk_id * q + min((int64_t)sk_id, rem);
+      last = (int64_t)dp_tiles * ipt + (sk_id + 1) * q + min((int64_t)sk_id + 1, rem);
     }
     if (p.mode == MODE_WS && p.cu_mask && p.cu_mask[pid] == 0) step = 1 << 30;  // masked out: nothing to do
+  }
+
+  // The XCD x slot queues over tiles [0, total): see next().  `raw`: the workgroup id the hardware gave out (its XCD
+  // and slot follow from it).
+  __device__ __forceinline__ bool queue_next(const GemmParams& p, int total, int raw, Work& w, int* s_bcast, int tid) {
+    const int X = p.num_xcds, S = p.counters_per_xcd;
+    const int xcd = raw % X, slot = (raw / X) % S;
+      if (tid < 64) {
+        const int lane = tid;
+        int found = -1, found_step = X * S;
+        for (int base = step; base < X * S && found < 0; base += 64) {
+          const int v = base + lane;
+          const bool valid = v < X * S;
+          const int qx = (xcd + v / S) % X;
+          const int qs = (slot + v % S) % S;
+          int qfirst, qcount;
+          ws_queue_range(WS_QUEUES, qx * S + qs, total, X, S, 0, qfirst, qcount);
+          const int bound = valid ? qcount : 0;
+          int32_t* ctr = p.counters + (qx * S + qs) * COUNTER_STRIDE;
+          const int seen = bound > 0 ? __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+          unsigned long long open = __ballot(bound > 0 && seen < bound);
+          while (open != 0 && found < 0) {
+            const int l = __builtin_ctzll(open);
+            int idx = 0;
+            if (lane == l) idx = atomicAdd(ctr, 1);
+            idx = __shfl(idx, l);
+            const int b = __shfl(bound, l), first = __shfl(qfirst, l);
+            if (idx < b) { found = first + idx; found_step = base + l; }
+            open &= open - 1;
+          }
+        }
+        if (lane == 0) { s_bcast[0] = found; s_bcast[1] = found_step; }
+      }
+      __syncthreads();
+      const int tile = s_bcast[0];
+      step = s_bcast[1];
+      __syncthreads();
+      if (tile < 0) return false;
+      plain_tile(p, tile, T::BM, T::BN, w.tc);
+      return true;
   }
 
   __device__ __forceinline__ bool next(const GemmParams& p, Work& w, int* s_bcast, int tid) {
@@ -1265,43 +1312,16 @@ struct Sched {
         plain_tile(p, tile, T::BM, T::BN, w.tc);
         return true;
       }
-      if (tid < 64) {
-        const int lane = tid;
-        int found = -1, found_step = X * S;
-        for (int base = step; base < X * S && found < 0; base += 64) {
-          const int v = base + lane;
-          const bool valid = v < X * S;
-          const int qx = (xcd + v / S) % X;
-          const int qs = (slot + v % S) % S;
-          int qfirst, qcount;
-          ws_queue_range(WS_QUEUES, qx * S + qs, p.total_tiles, X, S, 0, qfirst, qcount);
-          const int bound = valid ? qcount : 0;
-          int32_t* ctr = p.counters + (qx * S + qs) * COUNTER_STRIDE;
-          const int seen = bound > 0 ? __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
-          unsigned long long open = __ballot(bound > 0 && seen < bound);
-          while (open != 0 && found < 0) {
-            const int l = __builtin_ctzll(open);
-            int idx = 0;
-            if (lane == l) idx = atomicAdd(ctr, 1);
-            idx = __shfl(idx, l);
-            const int b = __shfl(bound, l), first = __shfl(qfirst, l);
-            if (idx < b) { found = first + idx; found_step = base + l; }
-            open &= open - 1;
-          }
-        }
-        if (lane == 0) { s_bcast[0] = found; s_bcast[1] = found_step; }
-      }
-      __syncthreads();
-      const int tile = s_bcast[0];
-      step = s_bcast[1];
-      __syncthreads();
-      if (tile < 0) return false;
-      plain_tile(p, tile, T::BM, T::BN, w.tc);
-      return true;
+      return queue_next(p, p.total_tiles, pid, w, s_bcast, tid);
     }
     if constexpr (!SK) return false;
-    // MODE_SK: data-parallel tiles first, then this workgroup's share of the Stream-K iterations
-    if (next_tile < dp_tiles) {
+    // MODE_SK: data-parallel tiles first (from the work-stealing queues when asked for, reference
+    // kernels/streamk_gemm_work_stealing.py:9-418), then this workgroup's share of the Stream-K iterations
+    if (ws_phase) {
+      if (queue_next(p, dp_tiles, sk_id, w, s_bcast, tid)) return true;
+      ws_phase = false;
+      step = 0;
+    } else if (p.sk_ws == 0 && next_tile < dp_tiles) {
       plain_tile(p, next_tile, T::BM, T::BN, w.tc);
       next_tile += G;
       return true;
@@ -1310,20 +1330,34 @@ struct Sched {
     // the head of the range's last tile) comes first and is published at once; the pieces that do
     // reach a tile's end finish that tile, adding what lower workgroups published long before.
     if (start >= last) return false;
-    const int ipt = p.k_iters;
+    const int unit = max(1, p.sk_unit);
+    const int ipt = p.k_iters / unit;
     const int tile = (int)((last - 1) / ipt);
     const int64_t tile_first = (int64_t)tile * ipt;
     const int64_t tile_end = tile_first + ipt;
     const int64_t begin = max(tile_first, start);
     plain_tile(p, tile, T::BM, T::BN, w.tc);
-    w.it0 = (int)(begin - tile_first);
-    w.it1 = (int)(last - tile_first);
+    w.it0 = (int)(begin - tile_first) * unit;
+    w.it1 = (int)(last - tile_first) * unit;
     w.kind = (last != tile_end) ? WK_SK_PUBLISH : WK_SK_OWNER;
     w.seg_begin = begin; w.tile_first = tile_first;
     last = begin;
     return true;
   }
 };
+
+// What the last workgroup of a Stream-K launch to leave does: advance the launch count the workspace keeps (every
+// workgroup has read it before it gets here) and rearm the work-stealing queues if the launch drew from them.
+__device__ __forceinline__ void sk_leave(const GemmParams& p, uint32_t epoch, int tid) {
+  if (p.mode != MODE_SK || tid != 0 || (p.epoch != EPOCH_ON_DEVICE && !p.sk_ws)) return;
+  const uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
+  if (done != gridDim.x - 1) return;
+  if (p.sk_ws)
+    for (int qi = 0; qi <= p.num_xcds * p.counters_per_xcd; ++qi)
+      __hip_atomic_store(p.counters + qi * COUNTER_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (p.epoch == EPOCH_ON_DEVICE) __hip_atomic_store(p.ctl + CTL_EPOCH, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // SK = false: data-parallel, work-stealing and grouped schedules (every work item is a whole tile).
 // SK = true: adds the Stream-K tail with its partial-tile publish / fixup paths.  Two kernels, so that
@@ -1417,14 +1451,7 @@ __global__ __launch_bounds__(T::THREADS, T::MINB) void gemm_kernel(const GemmPar
   }
   if constexpr (SK) {
     if (failed && li.tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
-    if (p.epoch == EPOCH_ON_DEVICE && p.mode == MODE_SK && li.tid == 0) {
-      // every workgroup has read the count before it gets here, so the last one to leave may advance it
-      const uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
-      if (done == gridDim.x - 1) {
-        __hip_atomic_store(p.ctl + CTL_EPOCH, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(p.ctl + CTL_DONE, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
+    sk_leave(p, epoch, li.tid);
   }
   if (!SK && p.mode == MODE_WS && li.tid == 0) {
     // the last workgroup to leave rearms the queues for the next launch

@@ -13,6 +13,17 @@ const void* w4_kernel(int dt) {
   return nullptr;
 }
 
+// the same kernels with the Stream-K tail
+const void* w4_kernel_sk(int dt) {
+  if (dt == DT_FP8) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP8>, true>;
+  if (dt == DT_E5M2) return (const void*)&gemm_kernel_w4<W4Tile<DT_E5M2>, true>;
+  if (dt == DT_FP4) return (const void*)&gemm_kernel_w4<W4Tile<DT_FP4>, true>;
+  if (dt == DT_BF16) return (const void*)&gemm_kernel_w4<W4Tile<DT_BF16>, true>;
+  if (dt == DT_F16) return (const void*)&gemm_kernel_w4<W4Tile<DT_F16>, true>;
+  if (dt == DT_I8) return (const void*)&gemm_kernel_w4<W4Tile<DT_I8>, true>;
+  return nullptr;
+}
+
 }  // namespace tb
 
 #ifdef W4_LAB_TS

@@ -12,7 +12,8 @@ struct Variant {
   int fast, stages;       // fast: vector/LDS-direct loaders (alignment + K multiple required)
   const void* kernel;     // __global__ void (*)(const GemmParams), whole-tile schedules
   const void* kernel_sk;  // same tile with the Stream-K tail (null: this variant has none)
-  int k_step_pairs;       // 1: hand-scheduled 4-wave kernel -- K must be an even number of K steps, at least four
+  int k_step_pairs;       // 1: hand-scheduled 4-wave kernel -- K must be an even number of K steps, at least four; with a
+                          // Stream-K tail a multiple of four (the K ranges of its pieces are cut at multiples of four steps)
 };
 
 template <class T>
@@ -24,6 +25,7 @@ constexpr Variant make_variant() {
 // The hand-scheduled 4-wave kernels of gemm_w4.h (256x256 tile, 128-byte K steps) are compiled in a
 // translation unit of their own (gemm_inst_w4.hip), which hands out their addresses.
 const void* w4_kernel(int dt);
+const void* w4_kernel_sk(int dt);
 template <int DT>
 using W4Tile = Tile<DT, 256, 256, 128, 2, 2, LAY_K, LAY_K, 1, true, 2>;
 // LDS of these kernels: two 64 KB stages, 16 KB of FP4 scale buffers, 1 KB per wave of epilogue scales,
@@ -33,7 +35,7 @@ constexpr int W4_LDS_BYTES = W4_EPS_OFFSET + 4096 + 16;
 template <class T>
 Variant make_variant_w4() {
   return Variant{T::DT, T::BM, T::BN, T::BK, T::ALAY, T::BLAY, T::WM, T::WN, T::THREADS, W4_LDS_BYTES, 1,
-                 1, T::STAGES, w4_kernel(T::DT), nullptr, 1};
+                 1, T::STAGES, w4_kernel(T::DT), w4_kernel_sk(T::DT), 1};
 }
 
 // defined one per translation unit

@@ -79,20 +79,21 @@ struct W4Lane {
   int sra, srb;          // FP4: tile rows whose scales this lane copies
 };
 
+// it0: first K step of the work item (a Stream-K piece starts inside the tile's K range)
 template <class T>
-__device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, W4TileArgs& t) {
+__device__ __forceinline__ void w4_tile_args(const GemmParams& p, const TileCtx& tc, int it0, const W4Lane& ln, W4TileArgs& t) {
   const int rva = tc.m_lim - tc.m0, rvb = tc.n_lim - tc.n0;
   const uint32_t sra = (uint32_t)p.a_sr * T::USZ, srb = (uint32_t)p.b_sr * T::USZ;   // row strides in bytes
-  t.A = p.A + (int64_t)tc.m0 * p.a_sr * T::USZ;
-  t.B = tc.B + (int64_t)tc.n0 * p.b_sr * T::USZ;
+  t.A = p.A + (int64_t)tc.m0 * p.a_sr * T::USZ + (int64_t)it0 * 128;
+  t.B = tc.B + (int64_t)tc.n0 * p.b_sr * T::USZ + (int64_t)it0 * 128;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     t.off[i] = (int)((uint32_t)min(i * 32 + ln.pa, rva - 1) * sra + ln.c16);
     t.off[8 + i] = (int)((uint32_t)min(i * 32 + ln.pb, rvb - 1) * srb + ln.c16);
   }
   if constexpr (T::DT == DT_FP4) {
-    t.mxa = p.mxa + (int64_t)tc.m0 * p.mxa_sr;
-    t.mxb = p.mxb + (int64_t)tc.n0 * p.mxb_sr;
+    t.mxa = p.mxa + (int64_t)tc.m0 * p.mxa_sr + it0 * 8;      // (eight E8M0 bytes per row and K step)
+    t.mxb = p.mxb + (int64_t)tc.n0 * p.mxb_sr + it0 * 8;
     t.sca = (uint32_t)min(ln.sra, rva - 1) * (uint32_t)p.mxa_sr;
     t.scb = (uint32_t)min(ln.srb, rvb - 1) * (uint32_t)p.mxb_sr;
   } else {
@@ -226,6 +227,113 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
   });
 }
 
+// ---- Stream-K pieces ---------------------------------------------------------------------------------------
+// A partial tile travels in the order the accumulators have it: MFMA tile t = 8 i + j of wave w is one 16-byte
+// value per lane at float offset ((w * 64 + t) * 64 + lane) * 4 of the workgroup's slot -- 1 KB per store, no
+// layout change on either side.  Device-scope (sc1) accesses: publisher and owner usually sit on different XCDs.
+template <class T>
+__device__ __forceinline__ void partial_store_w4(float* slot, int wave, int lane) {
+  const uint32_t off = (uint32_t)lane * 16u;
+  static_for<64>([&](auto TT) {
+    constexpr int t = decltype(TT)::value;
+    v4f v;
+    v[0] = acc_read<t * 4 + 0, T::DT == DT_I8>(); v[1] = acc_read<t * 4 + 1, T::DT == DT_I8>();
+    v[2] = acc_read<t * 4 + 2, T::DT == DT_I8>(); v[3] = acc_read<t * 4 + 3, T::DT == DT_I8>();
+    const float* base = slot + (size_t)(wave * 64 + t) * 256;
+    const uint32_t o = off;   // (assembly operands do not capture: name locals of this lambda)
+    // (the wait states behind the store: it still reads its data registers for a moment after it issues, and the
+    // compiler, which cannot see into the statement, lets the next accumulator read reuse them at once)
+    asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 sc1\n\ts_nop 1" : : "v"(o), "v"(v), "s"(base) : "memory");
+  });
+}
+
+// The tile's owner: its own sums plus the partial tiles of workgroups id_hi, id_hi - 1, ... (n of them, nearest
+// first: a fixed order), then acc * (sa*sb) + bias -> cast -> store with bounds.  poison: a partner did not
+// publish in time, the tile is stored as NaN.
+template <class T, int CT>
+__device__ __forceinline__ void epilogue_w4_owner(const GemmParams& p, const TileCtx& tc, const W4Lane& ln, int wave, int lane,
+                                                  int id_hi, int n, bool poison) {
+  const uint32_t off = (uint32_t)lane * 16u;
+  float sav[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = tc.m0 + ln.wm0 + i * 16 + ln.r;
+    sav[i] = (p.sa && m < tc.m_lim) ? p.sa[m] : 1.f;
+  }
+  static_for<4>([&](auto Q) {
+    constexpr int q = decltype(Q)::value;
+    // the 16 MFMA tiles (i, 2q) and (i, 2q + 1), i = 0..7, of this column group
+    v4f v[16];
+    static_for<16>([&](auto X) {
+      constexpr int x = decltype(X)::value;
+      constexpr int t = (x >> 1) * 8 + 2 * q + (x & 1);
+      v[x][0] = acc_read<t * 4 + 0, T::DT == DT_I8>(); v[x][1] = acc_read<t * 4 + 1, T::DT == DT_I8>();
+      v[x][2] = acc_read<t * 4 + 2, T::DT == DT_I8>(); v[x][3] = acc_read<t * 4 + 3, T::DT == DT_I8>();
+    });
+    const uint32_t o = off;   // (assembly operands do not capture: name locals of this lambda)
+    for (int k = 0; k < n; ++k) {
+      const float* slot = p.P + (size_t)(id_hi - k) * (256 * 256);
+      v4f part[16];
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const int t = (x >> 1) * 8 + 2 * q + (x & 1);
+        const float* base = slot + (size_t)(wave * 64 + t) * 256;
+        asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 sc1" : "=v"(part[x]) : "v"(o), "s"(base) : "memory");
+      }
+      // (the compiler does not know that these registers are written asynchronously)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        asm volatile("" : "+v"(part[x]));
+        v[x] += part[x];
+      }
+    }
+    const int ncol = tc.n0 + ln.wn0 + 32 * q + 8 * ln.g;
+    const int nvalid = tc.n_lim - ncol;
+    float sbv[8], bv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sbv[e] = (tc.sb && e < nvalid) ? tc.sb[ncol + e] : 1.f;
+      bv[e] = (p.bias && e < nvalid)
+                  ? load_as_f32(p.bias + (int64_t)(ncol + e) * p.bias_stride * (p.bias_type == DT_F32 ? 4 : 2), p.bias_type)
+                  : 0.f;
+    }
+    static_for<8>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      const int m = tc.m0 + ln.wm0 + i * 16 + ln.r;
+      if (m >= tc.m_lim || nvalid <= 0) return;
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = v[2 * i + (e >> 2)][e & 3];
+        if (p.sa) x = x * (sav[i] * sbv[e]);
+        if (p.bias) x = x + bv[e];
+        o[e] = poison ? __builtin_nanf("") : x;
+      }
+      if constexpr (CT == DT_F32) {
+        float* cp = (float*)p.C + ((int64_t)m * p.c_sm + (int64_t)ncol * p.c_sn);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (e < nvalid) cp[e * p.c_sn] = o[e];
+      } else {
+        uint16_t* cp = (uint16_t*)p.C + ((int64_t)m * p.c_sm + (int64_t)ncol * p.c_sn);
+        uint32_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if constexpr (CT == DT_F16) h[e] = __builtin_bit_cast(uint16_t, (_Float16)o[e]);
+          else h[e] = __builtin_bit_cast(uint16_t, (__bf16)o[e]);
+        }
+        if (p.c_line && nvalid >= 8) {
+          const v4i pk = {(int)(h[0] | (h[1] << 16)), (int)(h[2] | (h[3] << 16)), (int)(h[4] | (h[5] << 16)), (int)(h[6] | (h[7] << 16))};
+          *(v4i*)cp = pk;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (e < nvalid) cp[e * p.c_sn] = (uint16_t)h[e];
+        }
+      }
+    });
+  });
+}
+
 // operands every kind of K loop statement takes
 #define W4_COMMON_OPERANDS                                                                                              \
   [offc] "{v[192:207]}"(cur.off), [offn] "{v[208:223]}"(nxt.off), [fa] "{v[224:231]}"(fa), [A] "s"(sA), [B] "s"(sB),     \
@@ -237,7 +345,9 @@ __device__ __forceinline__ void epilogue_w4_fast(const GemmParams& p, const Tile
 __device__ unsigned long long w4_lab_ts[1024 * 32];
 #endif
 
-template <class T>
+// SK: the schedule may end in a Stream-K tail (pieces of a tile's K range, cut at multiples of four K steps:
+// GemmParams::sk_unit = 4), with the partial-tile exchange of gemm_kernel<T, true>.
+template <class T, bool SK = false>
 __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   static_assert(T::BM == 256 && T::BN == 256 && T::BKB == 128 && T::WM == 2 && T::WN == 2 && T::STAGES == 2, "fixed shape");
   static_assert(is_f8(T::DT) || T::DT == DT_FP4 || T::DT == DT_BF16 || T::DT == DT_F16 || T::DT == DT_I8, "element types with a generated K loop");
@@ -278,8 +388,13 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   }
   const uint32_t wl = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)wave * 1024u));
 
-  Sched<T, false> sched;
+  Sched<T, SK> sched;
   sched.init(p);
+  uint32_t epoch = p.epoch;
+  bool failed = false;
+  if constexpr (SK) {
+    if (p.epoch == EPOCH_ON_DEVICE) epoch = __hip_atomic_load(p.ctl + CTL_EPOCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  }
 #ifdef W4_LAB_TS
   int ts_n = 0;
   if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
@@ -290,7 +405,6 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   int first = 1;
   int nst = 0;             // 1: the previous tile's epilogue issued exactly 32 stores per wave (its fast path)
   uint32_t scbuf = 0;
-  const int kh = p.k_iters >> 1;
   // Fused epilogue: a full tile with bf16 output (and, for FP8, both scale vectors; for the other
   // kinds, none) is not stored by the code below but by the NEXT tile's K loop, which reads each
   // accumulator row block out just before its first K step overwrites it.  The last tile of a workgroup
@@ -311,10 +425,11 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     // the tile after this one: its first two K steps are requested during this tile's last two.  With
     // none left the copies read this tile's first steps again; nobody uses them.
     const bool have_next = sched.next(p, wnext, &s_bcast, tid);
-    if (!have_next) wnext.tc = w.tc;
+    if (!have_next) wnext = w;
     W4TileArgs cur, nxt;
-    w4_tile_args<T>(p, w.tc, ln, cur);
-    w4_tile_args<T>(p, wnext.tc, ln, nxt);
+    w4_tile_args<T>(p, w.tc, w.it0, ln, cur);
+    w4_tile_args<T>(p, wnext.tc, wnext.it0, ln, nxt);
+    const int kh = (w.it1 - w.it0) >> 1;
     const bool fast = p.c_line && !p.bias && p.c_type != DT_F32 && w.tc.m0 + 256 <= w.tc.m_lim && w.tc.n0 + 256 <= w.tc.n_lim &&
                       (!p.sa || (((uintptr_t)w.tc.sb & 15) == 0));
     const bool regs = (is_f8(T::DT) || T::DT == DT_I8) && fast && p.sa;    // the K loop copies this tile's scale vectors
@@ -381,7 +496,47 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
 #include "w4_clobbers_fp4.inc"
       );
     }
-    if (fast && fe_shape && have_next) {
+    bool sk_piece = false;
+    if constexpr (SK) {
+      if (w.kind == WK_SK_PUBLISH) {
+        // not the tile's last piece: publish the partial sums, tagged with this launch's epoch
+        sk_piece = true;
+        partial_store_w4<T>(p.P + (size_t)sched.sk_id * (256 * 256), wave, lane);
+        __builtin_amdgcn_s_waitcnt(0x0070);   // this wave's write-through stores have left the CU
+        __syncthreads();                      // ... and so have everybody else's
+        if (tid == 0) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+          __hip_atomic_store(p.flags + sched.sk_id, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else if (w.kind == WK_SK_OWNER) {
+        // the piece that ends the tile: wait for the pieces before it (lower workgroup ids only), add them, store
+        sk_piece = true;
+        int n = 0, nxt_id = sched.sk_id - 1;
+        for (int64_t b = w.seg_begin; b > w.tile_first; b -= sched.q + (nxt_id < sched.rem ? 1 : 0), --nxt_id) ++n;
+        if (tid == 0) {
+          int ok = 1;
+          for (int k = 0; k < n && ok; ++k) {
+            uint32_t spins = 0;
+            while (__hip_atomic_load(p.flags + (sched.sk_id - 1 - k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != epoch) {
+              if (++spins >= p.spin_limit) { ok = 0; break; }
+              __builtin_amdgcn_s_sleep(2);
+            }
+          }
+          s_bcast = ok;
+        }
+        __syncthreads();
+        const bool ok = s_bcast != 0;
+        __syncthreads();
+        if (!ok) failed = true;
+        if (p.c_type == DT_BF16) epilogue_w4_owner<T, DT_BF16>(p, w.tc, ln, wave, lane, sched.sk_id - 1, ok ? n : 0, !ok);
+        else if (p.c_type == DT_F16) epilogue_w4_owner<T, DT_F16>(p, w.tc, ln, wave, lane, sched.sk_id - 1, ok ? n : 0, !ok);
+        else epilogue_w4_owner<T, DT_F32>(p, w.tc, ln, wave, lane, sched.sk_id - 1, ok ? n : 0, !ok);
+      }
+    }
+    if (sk_piece) {
+      fe = 0;
+      nst = 0;      // (an unknown number of stores since the K loop)
+    } else if (fast && fe_shape && have_next) {
       // stored by the next tile's K loop
       fe = 1;
       cprev = (const uint8_t*)p.C + ((int64_t)(w.tc.m0 + ln.wm0) * p.c_sm + (w.tc.n0 + ln.wn0)) * 2;
@@ -410,7 +565,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     if (tid == 0 && blockIdx.x < 1024 && ts_n < 31) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
     ++ts_n;
 #endif
-    w.tc = wnext.tc;
+    w = wnext;
     have = have_next;
     first = 0;
   }
@@ -419,6 +574,10 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
 #ifdef W4_LAB_TS
   if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + 31] = __builtin_amdgcn_s_memrealtime();
 #endif
+  if constexpr (SK) {
+    if (failed && tid == 0) atomicExch(p.ctl + CTL_STATUS, 1u);
+    sk_leave(p, epoch, tid);
+  }
   if (p.mode == MODE_WS && tid == 0) {
     // the last workgroup to leave rearms the queues for the next launch
     uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);

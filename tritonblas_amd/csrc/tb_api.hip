@@ -146,11 +146,16 @@ std::vector<TileInfo> tile_infos(int dt) {
 // taken (measured, 64x64 bf16 tiles: 128x4096x4096 32 -> 22 us, 64x8192x8192 60 -> 39 us with four
 // stages; 2048^3 30 -> 35 us, which the rule avoids).
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast, int64_t total_tiles = 0,
-                            const tb_hw* hw = nullptr, bool need_sk = false, int64_t k = 0) {
+                            const tb_hw* hw = nullptr, bool need_sk = false, int64_t k = 0, bool out8 = false) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
-  // the hand-scheduled 4-wave kernels run K steps in pairs and have no Stream-K form
-  auto usable = [&](const Variant& x) { return !x.k_step_pairs || (!need_sk && k >= 4 * (int64_t)x.bk && k % (2 * (int64_t)x.bk) == 0); };
+  // the hand-scheduled 4-wave kernels run K steps in pairs (the pieces of a Stream-K tail in blocks of four) and
+  // have no 8-bit output path
+  auto usable = [&](const Variant& x) {
+    if (!x.k_step_pairs) return true;
+    if (out8 || (need_sk && !x.kernel_sk)) return false;
+    return k >= 4 * (int64_t)x.bk && k % ((need_sk ? 4 : 2) * (int64_t)x.bk) == 0;
+  };
   const int want = hooks().waves;
   if (want && fast)
     for (int i = 0; i < n; ++i)
@@ -223,6 +228,8 @@ struct Plan {
   size_t ws_need = 0, ws_flags_off = 0, ws_p_off = 0, ws_counters_off = 0;
 };
 
+bool is_streamk(int schedule) { return schedule == TB_SCHED_STREAMK || schedule == TB_SCHED_STREAMK_WS; }
+
 int kernel_occupancy(const Variant* v, const void* kernel) {
   static std::mutex mu;
   static std::vector<std::pair<const void*, int>> cache;
@@ -265,7 +272,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     std::memset(&pr, 0, sizeof(pr));
     pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
     pr.a_k_contiguous = alay == LAY_K; pr.b_k_contiguous = blay == LAY_K;
-    pr.streamk = j.schedule == TB_SCHED_STREAMK; pr.num_groups = j.num_groups;
+    pr.streamk = is_streamk(j.schedule); pr.num_groups = j.num_groups;
     auto infos = tile_infos(j.dt);
     int st = select_tile(pr, hw, infos.data(), (int)infos.size(), &sel);
     if (st != TB_OK) return st;
@@ -289,11 +296,10 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     // workgroups that have to be resident at once for a deeper-pipeline variant to be the better one:
     // all tiles, and for Stream-K the whole grid (the owners wait for the other segments' workgroups)
     int64_t at_once = ((j.M + bm - 1) / bm) * ((j.N + bn - 1) / bn);
-    if (j.schedule == TB_SCHED_STREAMK) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
+    if (is_streamk(j.schedule)) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
     if (j.num_groups > 0) at_once = 0;
-    // (the 4-wave kernels have no Stream-K form and no 8-bit output path)
-    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw,
-                     (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) || j.c_type == TB_FP8_E4M3 || j.c_type == TB_I8, j.K);
+    v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw, is_streamk(j.schedule) && j.num_groups == 0, j.K,
+                     j.c_type == TB_FP8_E4M3 || j.c_type == TB_I8);
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
@@ -343,7 +349,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.group_offsets = j.group_offsets; p.num_groups = j.num_groups;
   p.b_group_stride = j.b_group_stride; p.sb_group_stride = j.sb_group_stride;
 
-  const void* kern = (j.schedule == TB_SCHED_STREAMK && j.num_groups == 0) ? v->kernel_sk : v->kernel;
+  const void* kern = (is_streamk(j.schedule) && j.num_groups == 0) ? v->kernel_sk : v->kernel;
   {
     // a handful of rows against a K-major weight: the streaming kernel (no tiles, no workspace) when
     // the model expects it to beat the tile kernel of the requested schedule.  TB_NO_SKINNY=1 / TB_SKINNY=1
@@ -355,7 +361,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       std::memset(&pr, 0, sizeof(pr));
       pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
       pr.a_k_contiguous = pr.b_k_contiguous = 1;
-      const bool sk = j.schedule == TB_SCHED_STREAMK;
+      const bool sk = is_streamk(j.schedule);
       const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, v->minb, v->fast, v->stages};
       plan->skinny = estimate_streaming_us(pr, hw) < estimate_tile_us(pr, hw, ti, sk);
     }
@@ -407,8 +413,9 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if ((size_t)p.num_xcds * p.counters_per_xcd + 1 > WS_MAX_LINES) return TB_ERR_BAD_SCHEDULE;
     plan->ws_counters_off = WS_COUNTERS_OFF;
     plan->ws_need = WS_FLAGS_OFF;
-  } else if (j.schedule == TB_SCHED_STREAMK) {
+  } else if (is_streamk(j.schedule)) {
     p.mode = MODE_SK;
+    p.sk_unit = v->k_step_pairs ? 4 : 1;
     // (a requested grid larger than what is resident at once for the kernel that really runs -- the caller
     // sized it for another tile, e.g. the operands turned out to need the gather kernel -- gives way to
     // the library's own choice.  Correctness does not need residency: a tile's owner only waits for
@@ -437,6 +444,14 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       // which may be the hand-scheduled 4-wave form of this tile, ruled out above only for its lack of
       // a Stream-K tail (same tile, one workgroup per CU either way, bit-identical sums)
       p.mode = MODE_STATIC;
+      p.sk_unit = 0;
+      if (j.schedule == TB_SCHED_STREAMK_WS) {
+        // (the work-stealing launch of the same tiles; its workspace is the queue counters)
+        Job whole = j;
+        whole.schedule = TB_SCHED_WORK_STEALING;
+        whole.grid = 0;
+        return make_plan(whole, hw, need_device, plan);
+      }
       if (v->fast && j.c_type != TB_FP8_E4M3 && j.c_type != TB_I8) {
         const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K);
         if (w && w->k_step_pairs && w->bm == v->bm && w->bn == v->bn && w->bk == v->bk &&
@@ -447,6 +462,13 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
       plan->ws_flags_off = WS_FLAGS_OFF;
       plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
       plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
+      if (j.schedule == TB_SCHED_STREAMK_WS) {
+        // the whole tiles in front of the tail come from the XCD x slot queues (counters and flags never overlap)
+        p.sk_ws = 1;
+        p.counters_per_xcd = j.counters_per_xcd > 0 ? j.counters_per_xcd : ws_counters_per_xcd(total - p.sk_tiles);
+        if ((size_t)p.num_xcds * p.counters_per_xcd + 1 > WS_MAX_LINES) return TB_ERR_BAD_SCHEDULE;
+        plan->ws_counters_off = WS_COUNTERS_OFF;
+      }
     }
   } else {
     return TB_ERR_BAD_SCHEDULE;
@@ -555,7 +577,7 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
     if (p.mode == MODE_SK && j.epoch == 0) return TB_ERR_BAD_ARGUMENT;
     uint8_t* ws = (uint8_t*)j.workspace;
     p.ctl = (uint32_t*)ws;
-    if (p.mode == MODE_WS) p.counters = (int32_t*)(ws + plan.ws_counters_off);
+    if (p.mode == MODE_WS || p.sk_ws) p.counters = (int32_t*)(ws + plan.ws_counters_off);
     if (p.mode == MODE_SK) { p.flags = (uint32_t*)(ws + plan.ws_flags_off); p.P = (float*)(ws + plan.ws_p_off); }
   }
   void* args[] = {(void*)&p};
@@ -853,6 +875,27 @@ int tb_static_workspace_status(int* status, int clear) {
     if (hipMemcpy(at, &zero, 4, hipMemcpyHostToDevice) != hipSuccess) return TB_ERR_LAUNCH;
   }
   *status = (int)word;
+  return TB_OK;
+}
+
+int tb_gemm_launch_info(const tb_gemm_desc* desc, tb_launch_info* out) {
+  if (!out) return TB_ERR_NULL_POINTER;
+  Job j;
+  int st = job_from_gemm(desc, &j);
+  if (st != TB_OK) return st;
+  tb_hw hw;
+  const bool have_dev = current_hw(&hw) == TB_OK;
+  if (!have_dev) default_hw(&hw);
+  Plan plan;
+  st = make_plan(j, hw, have_dev, &plan);
+  if (st != TB_OK) return st;
+  std::memset(out, 0, sizeof(*out));
+  out->block_m = plan.v->bm; out->block_n = plan.v->bn; out->block_k = plan.v->bk;
+  out->waves = plan.v->threads / 64; out->four_wave = plan.v->k_step_pairs ? 1 : 0;
+  out->mode = plan.p.mode; out->grid = plan.grid; out->total_tiles = plan.p.total_tiles;
+  out->sk_tiles = plan.p.mode == MODE_SK ? plan.p.sk_tiles : 0;
+  out->sk_unit = plan.p.mode == MODE_SK ? std::max(1, plan.p.sk_unit) : 0;
+  out->sk_ws = plan.p.sk_ws; out->skinny = plan.skinny ? 1 : 0;
   return TB_OK;
 }
 

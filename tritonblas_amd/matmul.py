@@ -134,7 +134,8 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
         d.group_m, d.num_xcds = selector.group_m, selector.num_sms
         d.counters_per_xcd = selector.COUNTERS_PER_XCD
     d.schedule = schedule
-    if selector is not None and getattr(selector, "_total_cus", None) is not None and schedule != _lib.TB_SCHED_STREAMK:
+    streamk = schedule in (_lib.TB_SCHED_STREAMK, _lib.TB_SCHED_STREAMK_WS)
+    if selector is not None and getattr(selector, "_total_cus", None) is not None and not streamk:
         # a selector built for a CU partition sizes the launch (reference matmul.py:113: grid = N_CU):
         # as many workgroups as that many CUs hold at once; a mask (below) makes it one per mask entry
         d.grid = selector._N_CU * max(1, selector.waves_per_eu)
@@ -152,7 +153,7 @@ def _launch_gemm(a, b, c, selector, config, schedule, bias=None, a_scale=None, b
                 raise RuntimeError("tritonblas_amd: config.mask must be a contiguous int32 tensor on the GEMM's device")
             d.cu_mask, d.cu_mask_len = _ptr(mask), mask.numel()
             d.grid = 0
-    if schedule == _lib.TB_SCHED_STREAMK:
+    if streamk:
         if sk_grid is not None:
             d.grid = int(sk_grid)
         elif selector is not None and selector.streamk:
@@ -185,9 +186,14 @@ def persistent_matmul_lt(a, b, c, selector, config: Optional[MatmulConfig] = Non
 
 def streamk_matmul_lt(a, b, c, selector, config: Optional[MatmulConfig] = None, bias=None, sk_grid=None,
                       a_scale=None, b_scale=None, quantized: bool = False, work_stealing: bool = False):
-    """Stream-K launch (reference matmul.py:202-366).  ``work_stealing`` only changes the grid in the
-    reference (grid = CU count); here the Stream-K grid already fills the device."""
-    return _launch_gemm(a, b, c, selector, config, _lib.TB_SCHED_STREAMK, bias=bias, sk_grid=sk_grid,
+    """Stream-K launch (reference matmul.py:202-366).  ``work_stealing``: the whole tiles in front of the
+    Stream-K tail are drawn from the XCD x slot queues instead of being dealt out by workgroup id (reference
+    matmul.py:279-323, kernels/streamk_gemm_work_stealing.py); the tail itself is the same, and so are the
+    results.  A launch that shares the device with other work can run into the poll bound of the partial-tile
+    exchange (NaN tiles + the workspace's status word): callers in that situation should call
+    ``config.check()`` after synchronising."""
+    sched = _lib.TB_SCHED_STREAMK_WS if work_stealing else _lib.TB_SCHED_STREAMK
+    return _launch_gemm(a, b, c, selector, config, sched, bias=bias, sk_grid=sk_grid,
                         a_scale=a_scale if quantized else None, b_scale=b_scale if quantized else None)
 
 
