@@ -157,7 +157,9 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
     // one extra K segment of a tile costs its partial tile written through, polled for and added by the
     // owner, one after the other: ~1.5 us + the fp32 tile at ~10 GB/s (fitted on segment-count sweeps:
     // 32x128 tiles ~3 us, 128x128 tiles ~8 us, 256x256 tiles ~30 us per extra segment)
-    const double fix_us = 1.5 + area * 4.0 / 10e3;
+    // The 4-wave 256x256 kernels (256 threads) exchange partial tiles straight from the accumulators with 16 loads in
+    // flight per lane: ~12 us per extra segment (fitted: 2048x2048x16384 cut in four, FP8 92 us, bf16 137 us).
+    const double fix_us = 1.5 + area * 4.0 / 10e3 * ((v.threads == 256 && area >= 256 * 256) ? 0.4 : 1.0);
     const int slots = hw.n_cu * occ;
     const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu, std::max(t_thru, t_lat), fix_us);
     if (sk_grid_out) *sk_grid_out = grid;
