@@ -395,6 +395,12 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   if constexpr (SK) {
     if (p.epoch == EPOCH_ON_DEVICE) epoch = __hip_atomic_load(p.ctl + CTL_EPOCH, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
   }
+#ifdef W4_LAB_XCD_DELAY
+  // measurement build: the workgroups of the odd XCDs start (debug >> 8) * 8128 cycles late, so that the XCDs
+  // reach their tile changes (and the store bursts of the fused epilogues) at different times
+  if (blockIdx.x & 1)
+    for (int i = 0; i < (p.debug >> 8); ++i) __builtin_amdgcn_s_sleep(127);
+#endif
 #ifdef W4_LAB_TS
   int ts_n = 0;
   if (tid == 0 && blockIdx.x < 1024) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
