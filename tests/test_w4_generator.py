@@ -46,10 +46,16 @@ def test_program_shape(kind):
     g = gen.Gen(kind)
     parts = g.parts()
     per_step = 64 if kind in ("fp8", "e5m2") else 128
-    for name in ("first0", "first0_fe", "first1", "steady0", "steady1", "last0", "last1"):
+    for name in ("first0", "first0_fe", "first0_fe16", "first1", "steady0", "steady1", "last0", "last1"):
         assert sum(1 for o in parts[name] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")) == per_step, name
-    stores = [o for o in parts["first0_fe"] if not isinstance(o, gen.WaitVm) and o.text.startswith("global_store")]
-    assert len(stores) == 32
+    for fe in ("first0_fe", "first0_fe16"):
+        stores = [o for o in parts[fe] if not isinstance(o, gen.WaitVm) and o.text.startswith("global_store")]
+        assert len(stores) == 32
+    # the two fused epilogues differ in the conversion only
+    a = [o.text for o in parts["first0_fe"] if not isinstance(o, gen.WaitVm)]
+    b = [o.text for o in parts["first0_fe16"] if not isinstance(o, gen.WaitVm)]
+    assert len(a) == len(b) and all(x == y or (x.startswith("v_cvt_pk_bf16_f32") and y == x.replace("bf16", "f16")) or x.startswith(";")
+                                    for x, y in zip(a, b))
     assert not any(o.text.startswith("global_store") for o in parts["first0"] if not isinstance(o, gen.WaitVm))
     # the first K step starts every sum from zero, the others accumulate
     first = [o.text for o in parts["first0"] if not isinstance(o, gen.WaitVm) and o.text.startswith("v_mfma")]

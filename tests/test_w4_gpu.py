@@ -41,7 +41,7 @@ def _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=torch.bfloat16, bias=No
     a, b = aq.cuda(), bq.T.contiguous().cuda().T
     sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, out_dtype, a.device)
     sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, 128
-    c = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+    c = torch.full((m, n), float("nan"), device="cuda").to(out_dtype)
     cfg = tb.matmul_preamble(sel) if work_stealing else None
     persistent_matmul_lt(a, b, c, sel, cfg, bias=None if bias is None else bias.cuda(), a_scale=sa.cuda(), b_scale=sb.cuda(),
                          quantized=True, work_stealing=work_stealing)
@@ -235,6 +235,51 @@ def test_fused_epilogue(kind, bk, m, n, steps, grid, tb_option):
     assert torch.equal(again.view(torch.int16), fused.view(torch.int16))
 
 
+@pytest.mark.parametrize("kind", ["fp8", "f16"])
+@pytest.mark.parametrize("m,n,steps,grid", [(512, 768, 4, 1), (1280, 768, 6, 3), (1100, 1300, 8, 2), (4096, 4096, 4, 0)])
+def test_fused_epilogue_fp16_output(kind, m, n, steps, grid, tb_option):
+    """fp16 results take the fused epilogue too (its own conversion): the same bits as the compiled epilogue of
+    the same kernel and as the 8-wave kernel, and the oracle's values."""
+    import tritonblas_amd as tb
+    from tritonblas_amd.matmul import persistent_matmul_lt
+    bk = 128 if kind == "fp8" else 64
+    k = steps * bk
+    _say(f"fused epilogue, fp16 out, {kind} {m}x{n}x{k} grid {grid}")
+    if kind == "fp8":
+        aq, bq, sa, sb = _fp8_case(m, n, k, 87)
+        sa = sa * 0.05          # keep the results inside fp16's range
+        a, b = aq.cuda(), bq.T.contiguous().cuda().T
+        kw = dict(a_scale=sa.cuda(), b_scale=sb.cuda(), quantized=True)
+        want = OG.ref_gemm(aq, bq, torch.float32, a_scale=sa, b_scale=sb).half()
+        tol = TOL_Q
+    else:
+        g = torch.Generator().manual_seed(87)
+        a_cpu = (torch.randn(m, k, generator=g) * 0.5).half()
+        bt_cpu = (torch.randn(n, k, generator=g) * 0.5).half()
+        a, b = a_cpu.cuda(), bt_cpu.cuda().T
+        kw = {}
+        want = OG.ref_gemm(a_cpu, bt_cpu.T, torch.float32).half()
+        tol = 1e-3
+
+    def run():
+        sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, torch.float16, a.device)
+        sel._sel.block_m, sel._sel.block_n, sel._sel.block_k = 256, 256, bk
+        c = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+        persistent_matmul_lt(a, b, c, sel, None, **kw)
+        return c.cpu()
+    tb_option("grid", grid)
+    tb_option("waves", 24)
+    eight = run()
+    tb_option("waves", 22)
+    tb_option("lab", 4)
+    compiled = run()
+    tb_option("lab", 0)
+    fused = run()
+    assert OG.rel_fro_error(fused.float(), want.float()) <= tol
+    assert torch.equal(compiled.view(torch.int16), eight.view(torch.int16))
+    assert torch.equal(fused.view(torch.int16), compiled.view(torch.int16))
+
+
 def test_fused_epilogue_work_stealing(tb_option):
     """Tiles drawn from the work-stealing queues (which tile follows which is decided at run time) with
     two workgroups: same bits as the data-parallel launch."""
@@ -397,6 +442,26 @@ def test_a8w8_fp8_output_keeps_nan():
         assert torch.equal(got[100][~torch.isnan(got[100])], want[100][~torch.isnan(want[100])])
         fin = ~torch.isnan(want)
         torch.testing.assert_close(got[fin], want[fin], atol=2.0, rtol=0.2)
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 768, 512), (300, 500, 768), (1, 257, 512), (2048, 1280, 1024)])
+def test_fp8_four_wave_kernel_e4m3_output(m, n, k, tb_option):
+    """e4m3 results straight from the 4-wave kernel's accumulators (eight bytes per lane and row block): the same
+    bytes as the 8-wave kernel's, NaN kept, the reference's tolerance against the oracle."""
+    aq, bq, sa, sb = _fp8_case(m, n, k, 93)
+    sa = sa * 40.0
+    sa[0] = float("nan")
+    outs = {}
+    for waves in (22, 24):
+        outs[waves] = _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=torch.float8_e4m3fn)
+    want = OG.ref_gemm(aq, bq, torch.float8_e4m3fn, a_scale=sa, b_scale=sb)
+    assert torch.equal(outs[22].view(torch.uint8), outs[24].view(torch.uint8))
+    got = outs[22].float()
+    assert torch.isnan(got[0]).all() and not torch.isnan(got[1:]).any()
+    torch.testing.assert_close(got[1:], want.float()[1:], atol=2.0, rtol=0.2)
+    if m > 1:
+        same = (outs[22][1:].view(torch.uint8) == want[1:].view(torch.uint8)).float().mean().item()
+        assert same >= 0.99
 
 
 @pytest.mark.parametrize("m,n,k", [(256, 256, 256), (100, 300, 640), (512, 1024, 512)])

@@ -141,7 +141,25 @@ __device__ __forceinline__ void epilogue_w4(const GemmParams& p, const TileCtx& 
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = v[e] + bv[e];
       }
-      if constexpr (CT == DT_F32) {
+      if constexpr (CT == DT_FP8) {
+        // fp32 -> e4m3fn: clamp to the largest finite value (NaN stays NaN, as torch.clamp keeps it), round to
+        // nearest even; eight consecutive output columns are eight bytes
+        float cl[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) cl[e] = (v[e] != v[e]) ? v[e] : fminf(fmaxf(v[e], -448.f), 448.f);
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[0], cl[1], 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[2], cl[3], w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[4], cl[5], 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[6], cl[7], w1, true);
+        uint8_t* cp = p.C + ((int64_t)m * p.c_sm + (int64_t)n * p.c_sn);
+        if (p.c_vec && p.c_sn == 1 && nvalid >= 8 && (((uintptr_t)cp) & 7) == 0) {
+          *(uint2*)cp = uint2{(uint32_t)w0, (uint32_t)w1};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e < nvalid) cp[e * p.c_sn] = (uint8_t)((uint32_t)(e < 4 ? w0 : w1) >> (8 * (e & 3)));
+        }
+      } else if constexpr (CT == DT_F32) {
         float* cp = (float*)p.C + ((int64_t)m * p.c_sm + (int64_t)n * p.c_sn);
         if (p.c_line && nvalid >= 8) {
           const v4f lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
@@ -417,7 +435,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
   // always takes the code below.  An FP8 K loop copies its own tile's scale vectors into LDS for that.
   int fe = 0;                       // 1: the previous tile's sums are still in the accumulators
   const uint8_t* cprev = (const uint8_t*)p.C;   // C[first row of the wave's quarter][its first column] of that tile
-  const bool fe_shape = p.c_line && !p.bias && p.c_type == DT_BF16 && p.c_sm < (1 << 26) && (p.debug & 4) == 0 &&
+  const bool fe_shape = p.c_line && !p.bias && (p.c_type == DT_BF16 || p.c_type == DT_F16) && p.c_sm < (1 << 26) && (p.debug & 4) == 0 &&
                         ((is_f8(T::DT) || T::DT == DT_I8) == (p.sa != nullptr));
   // a lane's C offset from cprev, the same in every row block (rows of a row block are c_sm apart);
   // lane * 4; where the lane finds the scales of its rows 16 i + r and of its columns 32 q + 8 g + 0..7
@@ -543,8 +561,8 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
       fe = 0;
       nst = 0;      // (an unknown number of stores since the K loop)
     } else if (fast && fe_shape && have_next) {
-      // stored by the next tile's K loop
-      fe = 1;
+      // stored by the next tile's K loop (2: as fp16)
+      fe = p.c_type == DT_F16 ? 2 : 1;
       cprev = (const uint8_t*)p.C + ((int64_t)(w.tc.m0 + ln.wm0) * p.c_sm + (w.tc.n0 + ln.wn0)) * 2;
       nst = 0;
     } else {
@@ -564,7 +582,9 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
         }
       } else if (p.c_type == DT_BF16) epilogue_w4<T, DT_BF16>(p, w.tc, ln);
       else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
-      else epilogue_w4<T, DT_F32>(p, w.tc, ln);
+      else if (is_f8(T::DT) && p.c_type == DT_FP8) {
+        if constexpr (is_f8(T::DT)) epilogue_w4<T, DT_FP8>(p, w.tc, ln);
+      } else epilogue_w4<T, DT_F32>(p, w.tc, ln);
       nst = fast ? 1 : 0;
     }
 #ifdef W4_LAB_TS

@@ -205,7 +205,7 @@ class Gen:
         return Op(f"v_mfma_scale_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 3}], v[{a}:{a + 3}], {c}, "
                   f"v{self.scB(p, j)}, v{self.scA(p, i)} op_sel:[{ks},{ks},0] op_sel_hi:[0,0,0] cbsz:4 blgp:4")
 
-    def epilogue_block(self, i, tag):
+    def epilogue_block(self, i, tag, f16=False):
         """The previous tile's row block i: for each of its four column groups read eight sums, scale
         (FP8: acc * (sa[m] * sb[n]), the order the compiled epilogues use), round to bf16 pairs, store 16
         bytes.  Returns the instructions in order; the row pointer s[84:85] moves on afterwards."""
@@ -225,8 +225,9 @@ class Gen:
                     for x in range(4):
                         out.append(Op(f"v_mul_f32 v{s}, v{self.v_sa + i}, v{self.v_sb + q * 8 + h * 4 + x}"))
                         out.append(Op(f"v_mul_f32 v{e[x]}, v{e[x]}, v{s}"))
-                out.append(Op(f"v_cvt_pk_bf16_f32 v{pk[2 * h]}, v{e[0]}, v{e[1]}"))
-                out.append(Op(f"v_cvt_pk_bf16_f32 v{pk[2 * h + 1]}, v{e[2]}, v{e[3]}"))
+                cvt = "v_cvt_pk_f16_f32" if f16 else "v_cvt_pk_bf16_f32"
+                out.append(Op(f"{cvt} v{pk[2 * h]}, v{e[0]}, v{e[1]}"))
+                out.append(Op(f"{cvt} v{pk[2 * h + 1]}, v{e[2]}, v{e[3]}"))
             out.append(Op(f"global_store_dwordx4 v{self.v_coff}, v[{pk[0]}:{pk[3]}], s[{S_CROW}:{S_CROW + 1}] offset:{q * 64}", tag))
         out.append(Op(f"s_add_u32 s{S_CROW}, s{S_CROW}, %[cstep]"))
         out.append(Op(f"s_addc_u32 s{S_CROW + 1}, s{S_CROW + 1}, 0"))
@@ -266,8 +267,8 @@ class Gen:
         (oldest first, one set of destination registers each)."""
         nm = self.nm
         total = 8 * nm
-        first0 = flavor in ("first0", "first0_fe")
-        fe = flavor == "first0_fe"
+        first0 = flavor in ("first0", "first0_fe", "first0_fe16")
+        fe = flavor in ("first0_fe", "first0_fe16")
         eb = self.earlyb
         # early: the next step's B fragments 0..3 (and E8M0 scales) are read between X and Y instead of behind Y
         early = eb and prefetch and not fe
@@ -304,7 +305,7 @@ class Gen:
             # fused epilogue: row block 0 in front of the first MFMA, the others spread over row blocks 0..4:
             # block k is done before slot 5 nm k / 7 <= nm k, where its accumulators are overwritten, and
             # everything is done before the fragments of step 1 arrive in the registers used here
-            blocks = [self.epilogue_block(i, ("ST", 0)) for i in range(8)]
+            blocks = [self.epilogue_block(i, ("ST", 0), flavor == "first0_fe16") for i in range(8)]
             pre[0] += blocks[0]
             rest = [o for b in blocks[1:] for o in b]
             for n, o in enumerate(rest):
@@ -316,7 +317,7 @@ class Gen:
         xs = nm + self.xoff
         tail0 = 5 * nm + self.yoff
         # X: history keys of the waits (the counts are worked out by replay, see solve)
-        keys = {"steady": ["s"], "first0": ["a", "b", "c"], "first0_fe": ["d"], "first1": ["a", "b", "c", "d"]}[flavor]
+        keys = {"steady": ["s"], "first0": ["a", "b", "c"], "first0_fe": ["d"], "first0_fe16": ["d"], "first1": ["a", "b", "c", "d"]}[flavor]
         keys_x = ["s", "f"] if (flavor == "steady" and p == 0 and nsc) else keys
         wx = WaitVm(("XB", -1) if early else ("Y", -2), keys_x)
         pre[xs] += [Op("s_waitcnt lgkmcnt(0)"), wx, Op("s_barrier")]
@@ -495,6 +496,8 @@ class Gen:
         # (step 0 of a tile follows the entry reads: exactly those may be in flight)
         P["first0"] = self.step(0, False, True, "first0", self.read_dests(P["entry"]))
         P["first0_fe"] = self.step(0, False, True, "first0_fe", self.read_dests(P["entry_fe"] + P["entry"]))
+        # (the same with fp16 results: %[fe] = 2)
+        P["first0_fe16"] = self.step(0, False, True, "first0_fe16", self.read_dests(P["entry_fe"] + P["entry"]))
         P["first1"] = self.step(1, False, True, "first1")
         P["steady0"] = self.step(0, False, True)
         P["steady1"] = self.step(1, False, True)
@@ -580,7 +583,8 @@ class Gen:
             out += ["s_cmp_eq_u32 %[fe], 0", "s_cbranch_scc1 W4_NOSC%="] + T("entry_fe") + ["W4_NOSC%=:"]
         out += T("entry")
         out += ["s_cmp_lg_u32 %[fe], 0", "s_cbranch_scc1 W4_FE%="]
-        out += T("first0") + ["s_branch W4_FIRST1%=", "W4_FE%=:"] + T("first0_fe") + ["W4_FIRST1%=:"] + T("first1")
+        out += T("first0") + ["s_branch W4_FIRST1%=", "W4_FE%=:", "s_cmp_eq_u32 %[fe], 2", "s_cbranch_scc1 W4_FE16%="]
+        out += T("first0_fe") + ["s_branch W4_FIRST1%=", "W4_FE16%=:"] + T("first0_fe16") + ["W4_FIRST1%=:"] + T("first1")
         out += [f"s_sub_u32 s{S_CNT}, %[kh], 2", f"s_cmp_eq_u32 s{S_CNT}, 0", "s_cbranch_scc1 W4_LAST%=", "W4_LOOP%=:"]
         out += T("steady0") + T("steady1")
         out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_lg_u32 s{S_CNT}, 0", "s_cbranch_scc1 W4_LOOP%=", "W4_LAST%=:"]
@@ -615,9 +619,9 @@ class Gen:
                     elif o.vm is not None:
                         q.append((o.vm[0], o.vm[1] + step))
 
-        def tile(base, ksteps, hist0):
+        def tile(base, ksteps, hist0, fe_part="first0_fe"):
             """parts of one tile whose step 0 is number `base`"""
-            t = [("first0_fe" if hist0 == "d" else "first0", base, hist0), ("first1", base + 1, hist0)]
+            t = [(fe_part if hist0 == "d" else "first0", base, hist0), ("first1", base + 1, hist0)]
             h = "f"
             for it in range(2, ksteps - 2, 2):
                 t += [("steady0", base + it, h), ("steady1", base + it + 1, "s")]
@@ -626,9 +630,9 @@ class Gen:
             return t
 
         for k in (4, 6, 8, 10):
-            for hist, nstores in (("b", NST), ("c", 0), ("c", 50), ("d", 0)):
+            for hist, nstores, fe_part in (("b", NST, None), ("c", 0, None), ("c", 50, None), ("d", 0, "first0_fe"), ("d", 0, "first0_fe16")):
                 seq = [("prologue", 0, "a")] + tile(0, k, "a")
-                seq += [("cstores", k, nstores)] + tile(k, k, hist)
+                seq += [("cstores", k, nstores)] + tile(k, k, hist, fe_part)
                 seq += [("cstores", 2 * k, NST)] + tile(2 * k, k, "b")
                 run(seq)
 

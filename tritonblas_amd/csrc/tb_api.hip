@@ -146,14 +146,14 @@ std::vector<TileInfo> tile_infos(int dt) {
 // taken (measured, 64x64 bf16 tiles: 128x4096x4096 32 -> 22 us, 64x8192x8192 60 -> 39 us with four
 // stages; 2048^3 30 -> 35 us, which the rule avoids).
 const Variant* find_variant(int dt, int bm, int bn, int bk, int alay, int blay, int fast, int64_t total_tiles = 0,
-                            const tb_hw* hw = nullptr, bool need_sk = false, int64_t k = 0, bool out8 = false) {
+                            const tb_hw* hw = nullptr, bool need_sk = false, int64_t k = 0, int out8 = 0) {
   const Variant* v; int n;
   variant_table(dt, &v, &n);
-  // the hand-scheduled 4-wave kernels run K steps in pairs (the pieces of a Stream-K tail in blocks of four) and
-  // have no 8-bit output path
+  // the hand-scheduled 4-wave kernels run K steps in pairs (the pieces of a Stream-K tail in blocks of four); they
+  // store e4m3 results (out8 = 1) from whole tiles only and int8 results (out8 = 2) not at all
   auto usable = [&](const Variant& x) {
     if (!x.k_step_pairs) return true;
-    if (out8 || (need_sk && !x.kernel_sk)) return false;
+    if (out8 == 2 || (out8 == 1 && need_sk) || (need_sk && !x.kernel_sk)) return false;
     return k >= 4 * (int64_t)x.bk && k % ((need_sk ? 4 : 2) * (int64_t)x.bk) == 0;
   };
   const int want = hooks().waves;
@@ -299,7 +299,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (is_streamk(j.schedule)) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
     if (j.num_groups > 0) at_once = 0;
     v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw, is_streamk(j.schedule) && j.num_groups == 0, j.K,
-                     j.c_type == TB_FP8_E4M3 || j.c_type == TB_I8);
+                     j.c_type == TB_I8 ? 2 : (j.c_type == TB_FP8_E4M3 ? 1 : 0));
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
@@ -452,8 +452,8 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
         whole.grid = 0;
         return make_plan(whole, hw, need_device, plan);
       }
-      if (v->fast && j.c_type != TB_FP8_E4M3 && j.c_type != TB_I8) {
-        const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K);
+      if (v->fast && j.c_type != TB_I8) {
+        const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K, j.c_type == TB_FP8_E4M3 ? 1 : 0);
         if (w && w->k_step_pairs && w->bm == v->bm && w->bn == v->bn && w->bk == v->bk &&
             std::max(1, std::min(w->minb, hw.lds_bytes / w->lds_bytes)) == occ)
           v = w;
