@@ -150,6 +150,10 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
     if (whole <= 2 * (int64_t)hw.n_cu) t_lat *= 0.67;
     else if (whole <= 3 * (int64_t)hw.n_cu) t_lat *= 0.85;
   }
+  // the FP8 128x128 tile runs with four copy stages while every tile has a CU of its own
+  if (v.bm == 128 && v.bn == 128 && pr.num_groups == 0 && pr.a_type == TB_FP8_E4M3 &&
+      cdiv(pr.m, v.bm) * cdiv(pr.n, v.bn) <= (int64_t)hw.n_cu)
+    t_lat *= 0.67;
   const double t_tile = area >= 256 * 256 ? 12.0 : (area >= 128 * 128 ? 4.0 : 3.0);
 
   double us;
