@@ -36,6 +36,13 @@ def test_fast_compiled_epilogues(kind):
     replay(kind, 512, 512, ks, [(0, 0), (256, 0), (0, 256)], c_bf16=False)
 
 
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "bf16"])
+def test_stream_k_pieces(kind):
+    """a work list as the Stream-K schedule deals it out: whole tiles, then pieces of a tile's K range (multiples of
+    four K steps) whose copies start inside the operand rows -- including the look-ahead into the next piece"""
+    replay(kind, 512, 512, 16, [(0, 0), (256, 0, 8, 16), (0, 256, 4, 12), (256, 256, 0, 4), (256, 256)])
+
+
 def test_single_tile_workgroup():
     for kind in ("fp8", "fp4"):
         replay(kind, 256, 256, _steps(kind)[0], [(0, 0)])

@@ -118,10 +118,11 @@ class Wave:
     # ---- operand restatement of gemm_w4.h ------------------------------------------------------------------
     def tile_args(self, t):
         p = self.prob
-        m0, n0 = t
+        m0, n0 = t[:2]
+        it0 = t[2] if len(t) > 2 else 0          # a Stream-K piece starts at K step it0 of its tile
         rva, rvb = min(256, p.m - m0), min(256, p.n - n0)
-        a = {"A": p.A.base + m0 * p.A.stride, "B": p.B.base + n0 * p.B.stride,
-             "mxa": p.mxa.base + m0 * p.mxa.stride, "mxb": p.mxb.base + n0 * p.mxb.stride, "rva": rva, "rvb": rvb}
+        a = {"A": p.A.base + m0 * p.A.stride + it0 * 128, "B": p.B.base + n0 * p.B.stride + it0 * 128,
+             "mxa": p.mxa.base + m0 * p.mxa.stride + it0 * 8, "mxb": p.mxb.base + n0 * p.mxb.stride + it0 * 8, "rva": rva, "rvb": rvb}
         off = []
         for i in range(8):
             off.append(np.minimum(i * 32 + self.pa, rva - 1) * p.A.stride + self.c16)
@@ -141,10 +142,10 @@ class Wave:
         S, V = self.S, self.V
         for k, v in (("A", cur["A"]), ("B", cur["B"]), ("An", nxt["A"]), ("Bn", nxt["B"]), ("mxa", cur["mxa"]), ("mxb", cur["mxb"]),
                      ("mxan", nxt["mxa"]), ("mxbn", nxt["mxb"]), ("wl", LDS0 + self.wave * 1024),
-                     ("kh", p.ksteps // 2), ("first", first), ("nst", nst), ("fe", fe), ("cprev", cprev),
+                     ("kh", ((tiles[ti][3] - tiles[ti][2]) if len(tiles[ti]) > 2 else p.ksteps) // 2), ("first", first), ("nst", nst), ("fe", fe), ("cprev", cprev),
                      ("cstep", p.C.stride * 16), ("scbuf", scbuf)):
             S[f"%[{k}]"] = v
-        m0, n0 = tiles[ti]
+        m0, n0 = tiles[ti][:2]
         whole = m0 + 256 <= p.m and n0 + 256 <= p.n
         regs = p.scaled and whole
         S["%[sap]"] = p.sa.base + 4 * (m0 + self.wm0) if regs else cur["A"]
@@ -268,7 +269,7 @@ class Wave:
 
     # ---- what a fragment read must have fetched -----------------------------------------------------------------------
     def expect_rows(self, space, t, tile):
-        m0, n0 = self.prob.tiles[tile]
+        m0, n0 = self.prob.tiles[tile][:2]
         if space in ("A", "mxa"):
             return np.minimum(m0 + self.wm0 + 16 * t + self.r, self.prob.m - 1)
         rows = np.array([b_tile_row(int(x)) for x in (self.wn0 + 16 * t + self.r)])
@@ -371,7 +372,7 @@ class Wave:
         voff = self.vval("v" + m.group(1))
         self.vmq.append({"done": False, "lds": []})
         p = self.prob
-        m0, n0 = p.tiles[prev_tile]
+        m0, n0 = p.tiles[prev_tile][:2]
         for l in range(64):
             addr = base + int(voff[l])
             loc = p.C.locate(addr, 16)
@@ -463,7 +464,7 @@ class Wave:
     def note_eps(self, dst, got, prev_tile):
         """epilogue scales read back: the wave's rows 16 i + r of sa and columns 32 q + 8 g + 4 h + 0..3 of sb of the PREVIOUS tile"""
         p = self.prob
-        m0, n0 = p.tiles[prev_tile]
+        m0, n0 = p.tiles[prev_tile][:2]
         regs = sorted(self.gen.Gen._vregs(dst))
         for l in range(64):
             lane, _ = got[l]
@@ -489,7 +490,7 @@ class Group:
         for wv in range(4):
             self.waves.append(Wave(gen, prob, wv, self))
 
-    def run(self, lines, tile, prev_tile):
+    def run(self, lines, tile, prev_tile, first_step=0):
         labels = {l[:-1]: n for n, l in enumerate(lines) if l.endswith(":")}
         pc, kstep = 0, None
         while pc < len(lines):
@@ -499,7 +500,7 @@ class Group:
                 continue
             if t.startswith(";"):
                 if "K step" in t:
-                    kstep = 0 if kstep is None else kstep + 1
+                    kstep = first_step if kstep is None else kstep + 1
                     for w in self.waves:
                         w.step = (tile, kstep)
                 continue
@@ -517,7 +518,8 @@ class Group:
 
 
 def replay(kind, m, n, ksteps, tiles, c_bf16=True, pad=0, env=None):
-    """Runs the generated program of `kind` over `tiles` (list of (m0, n0)) for the four waves of a workgroup, the
+    """Runs the generated program of `kind` over `tiles` (list of (m0, n0), or (m0, n0, it0, it1) for a Stream-K
+    piece that covers K steps [it0, it1) of its tile) for the four waves of a workgroup, the
     way the loop of gemm_kernel_w4 would (history flags, fused or compiled epilogues).  Raises Fail on the first
     violation; returns the number of MFMAs checked."""
     gen = load_generator()
@@ -539,22 +541,24 @@ def replay(kind, m, n, ksteps, tiles, c_bf16=True, pad=0, env=None):
     checked = 0
     first, nst, fe, scbuf = 1, 0, 0, 0
     cprev = [prob.C.base] * 4
-    for ti, (m0, n0) in enumerate(tiles):
+    for ti, item in enumerate(tiles):
+        m0, n0 = item[:2]
+        piece = len(item) > 2          # a Stream-K piece (K steps [it0, it1)): its sums leave through compiled code
         have_next = ti + 1 < len(tiles)
         whole = m0 + 256 <= m and n0 + 256 <= n
-        fast = whole
+        fast = whole and not piece
         fe_shape = c_bf16
         before = []
         for w in grp.waves:
             w.bind(ti, first, nst, fe, cprev[w.wave], scbuf)
             before.append(dict(w.stores))
-        grp.run(lines, ti, ti - 1)
-        checked += 4 * ksteps * (64 if kind in ("fp8", "e5m2") else 128)
+        grp.run(lines, ti, ti - 1, item[2] if piece else 0)
+        checked += 4 * ((item[3] - item[2]) if piece else ksteps) * (64 if kind in ("fp8", "e5m2") else 128)
         scbuf = grp.waves[0].S["%[scbuf]"]
         for w in grp.waves:
             if fe:
                 # the wave's quarter of the previous tile: every 16 bytes exactly once
-                pm, pn = tiles[ti - 1]
+                pm, pn = tiles[ti - 1][:2]
                 for row in range(pm + w.wm0, pm + w.wm0 + 128):
                     for col in range(2 * (pn + w.wn0), 2 * (pn + w.wn0 + 128), 16):
                         a = prob.C.base + row * prob.C.stride + col
