@@ -257,9 +257,26 @@ typedef struct tb_grouped_gemm_desc {
                                  (rounds of tall tiles against rounds of short ones) and split only
                                  when that is cheaper; off when block_m is forced.  -1: one launch.
                                  The split needs k % 256 == 0 and a tall (>= 128-row) tile.            */
+  int32_t streamk;            /* 1: the tiles that do not fill whole rounds of the grid are cut into K ranges
+                                 (Stream-K, as kernels/streamk_gemm.py:160-384 does for one matrix) whenever the
+                                 tile table -- known only on the device -- makes that cheaper than one more
+                                 round; taken by the 256x256 four-wave kernel when k is a multiple of 512, ignored
+                                 otherwise.  Needs the workspace below; results then differ from streamk = 0
+                                 in the summation order of the cut tiles only.  0: whole tiles only.      */
+  uint32_t epoch;             /* as tb_gemm_desc.epoch; TB_EPOCH_ON_DEVICE: the workspace counts       */
+  uint32_t spin_limit;        /* as tb_gemm_desc.spin_limit                                           */
+  void* workspace;            /* tb_grouped_workspace_bytes() bytes, 256-byte aligned, zeroed once       */
+  size_t workspace_bytes;
 } tb_grouped_gemm_desc;
 
 int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* desc, void* stream);
+/* Workspace a streamk = 1 call with this descriptor needs (0: none, the launch runs whole tiles only). */
+size_t tb_grouped_workspace_bytes(const tb_grouped_gemm_desc* desc);
+/* Host-side evaluation of the rule the grouped kernel applies on the device: of a table of total_tiles tiles
+ * with k_units K units each (a unit = unit_steps K steps) on a grid of `grid` workgroups, how many tiles at
+ * the end are cut into K ranges; fix_steps = what an extra piece of a tile costs its owner, in K steps.  For
+ * tests; no counterpart in the reference. */
+int tb_streamk_tail_tiles(int32_t total_tiles, int32_t grid, int32_t k_units, int32_t unit_steps, int32_t fix_steps);
 
 /* ---- MXFP4 quantisation (replaces dynamic_mxfp4_quant, utils.py:743-789), optionally preceded
  *      by a 32-point blockwise Hadamard rotation along k (no counterpart in the reference) ------- */

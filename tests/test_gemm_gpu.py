@@ -727,3 +727,84 @@ def test_grouped_a8w8(counts):
         c2 = torch.empty_like(c)
         tb.grouped_matmul_a8w8(aq[rows].cuda(), wq[perm].cuda(), sa[rows].cuda(), sw[perm].cuda(), c2, off2.cuda())
         assert torch.equal(c2.cpu(), c.cpu()[rows])
+
+
+def _grouped_problem(counts, n, k, seed):
+    E, m = len(counts), sum(counts)
+    offsets = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)
+    a = torch.randn(m, k, generator=torch.Generator().manual_seed(seed)).bfloat16()
+    w = torch.randn(E, n, k, generator=torch.Generator().manual_seed(10000 + seed)).bfloat16()
+    aq, sa = OG.quantize_per_channel_fp8(a, axis=1)
+    wq, sw = OG.quantize_per_channel_fp8(w, axis=2)
+    return offsets, aq, wq, sa, sw
+
+
+@pytest.mark.parametrize("fix", [1, 64])
+@pytest.mark.parametrize("grid", [8, 5, 12])
+@pytest.mark.parametrize("counts", [[300, 0, 700, 24], [1, 255, 256, 257, 0, 0, 31, 224], [1024], [256, 256]])
+def test_grouped_streamk_tail(counts, grid, fix, tb_option):
+    """The tiles that do not fill whole rounds of the grid run as K ranges (Stream-K) on the 4-wave kernel: C
+    (NaN before) holds the oracle's values, the whole tiles are bit-identical to the launch without a tail, two
+    launches in a row share one workspace without a reset, and the configurations in which the device-side rule
+    must cut tiles show published partial tiles in the workspace.  fix: what the rule charges per extra piece of a
+    tile, in K steps (1: it cuts whenever a round is not full; 64: the library's value, which at this small K never cuts)."""
+    import tritonblas_amd as tb
+    from tritonblas_amd import _lib
+    from tritonblas_amd.config import MatmulConfig
+    _say(f"grouped streamk tail counts={counts} grid={grid} fix={fix}")
+    n, k = 512, 2048
+    tb_option("grid", grid)
+    tb_option("grp_sk_fix", fix)
+    offsets, aq, wq, sa, sw = _grouped_problem(counts, n, k, 24)
+    want = OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True)
+    args = (aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda())
+    m = sum(counts)
+    plain = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(*args, plain, offsets.cuda(), 256, 256, 128, small_rows=-1, enable_streamk=False)
+    cfg = MatmulConfig(device=plain.device, workspace=None)
+    c = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(*args, c, offsets.cuda(), 256, 256, 128, small_rows=-1, enable_streamk=True, config=cfg)
+    assert cfg.status() == 0
+    _check(c.cpu(), want, torch.bfloat16, TOL_Q)
+    tiles = sum((r + 255) // 256 for r in counts) * (n // 256)
+    launched = min(grid, ((m + 255) // 256 + len(counts)) * (n // 256))   # (the host only knows a bound of the table's length)
+    cut = _lib.load().tb_streamk_tail_tiles(tiles, launched, k // 512, 4, fix)
+    _, flags_off = _lib.workspace_layout()
+    flags = cfg.workspace[flags_off:flags_off + 4 * grid].view(torch.int32).cpu()
+    assert (int(flags.abs().sum()) > 0) == (cut > 0), (tiles, cut, flags)
+    # whole tiles are the table's first tiles: expert by expert, row block fastest
+    t, same = 0, 0
+    for e, rows in enumerate(counts):
+        mb = (rows + 255) // 256
+        for local in range(mb * (n // 256)):
+            if t < tiles - cut:
+                r0 = int(offsets[e]) + (local % mb) * 256
+                r1 = min(r0 + 256, int(offsets[e + 1]))
+                c0 = (local // mb) * 256
+                assert torch.equal(c[r0:r1, c0:c0 + 256], plain[r0:r1, c0:c0 + 256]), (e, local)
+                same += 1
+            t += 1
+    assert same == tiles - cut
+    # the same workspace again, other row counts, no reset
+    counts2 = list(reversed(counts))
+    offsets2, aq2, wq2, sa2, sw2 = _grouped_problem(counts2, n, k, 25)
+    c2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb.grouped_matmul_a8w8(aq2.cuda(), wq2.cuda(), sa2.cuda(), sw2.cuda(), c2, offsets2.cuda(), 256, 256, 128, small_rows=-1,
+                           enable_streamk=True, config=cfg)
+    assert cfg.status() == 0
+    _check(c2.cpu(), OG.ref_grouped_gemm_fp8(aq2, wq2, sa2, sw2, offsets2, return_fp32=True), torch.bfloat16, TOL_Q)
+
+
+def test_grouped_streamk_default_two_launch_plan(tb_option):
+    """Default plan (the device chooses between one and two launches) with the Stream-K tail on (the workspace is the
+    package's per-stream one): oracle values in every row."""
+    import tritonblas_amd as tb
+    _say("grouped streamk tail, default plan")
+    tb_option("grid", 6)
+    counts, n, k = [520, 30, 0, 300, 257], 512, 1024
+    offsets, aq, wq, sa, sw = _grouped_problem(counts, n, k, 26)
+    c = torch.full((sum(counts), n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tb_option("grp_sk_fix", 2)
+    for _ in range(2):
+        tb.grouped_matmul_a8w8(aq.cuda(), wq.cuda(), sa.cuda(), sw.cuda(), c, offsets.cuda(), enable_streamk=True)
+    _check(c.cpu(), OG.ref_grouped_gemm_fp8(aq, wq, sa, sw, offsets, return_fp32=True), torch.bfloat16, TOL_Q)

@@ -14,7 +14,7 @@ def _say(*a):
     print(*a, flush=True)
 
 
-@pytest.mark.parametrize("mode", ["streamk", "work_stealing", "persistent"])
+@pytest.mark.parametrize("mode", ["streamk", "work_stealing", "persistent", "streamk+work_stealing"])
 def test_python_launch_replays(mode):
     import tritonblas_amd as tb
     m, n, k = 512, 768, 4096
@@ -23,10 +23,10 @@ def test_python_launch_replays(mode):
     a = (torch.randn(m, k, device="cuda", generator=g) * 0.5).bfloat16()
     b = (torch.randn(k, n, device="cuda", generator=g) * 0.5).bfloat16()
     c = torch.zeros(m, n, dtype=torch.bfloat16, device="cuda")
-    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, c.dtype, a.device, streamk=mode == "streamk")
+    sel = tb.OrigamiMatmulSelector(m, n, k, a.dtype, b.dtype, c.dtype, a.device, streamk="streamk" in mode)
     cfg = tb.matmul_preamble(sel)
     cfg_eager = tb.matmul_preamble(sel)
-    kw = dict(enable_streamk=mode == "streamk", work_stealing=mode == "work_stealing")
+    kw = dict(enable_streamk="streamk" in mode, work_stealing="work_stealing" in mode)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -48,7 +48,7 @@ def test_python_launch_replays(mode):
         assert torch.equal(c.view(torch.int16), want.view(torch.int16)), f"replay {rep}"
         ref = (a.float() @ b.float())
         assert ((c.float() - ref).norm() / ref.norm()).item() <= 2e-3
-    if mode == "streamk":
+    if "streamk" in mode:
         assert cfg.status() == 0
 
 

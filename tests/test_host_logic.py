@@ -5,6 +5,7 @@ import os
 import re
 
 import pytest
+import numpy as np
 import torch
 
 from oracle import selector as O
@@ -413,3 +414,78 @@ def test_matmul_fp4_refuses_wrong_element_sizes_and_scale_shapes():
         tb.matmul_fp4(a.to(torch.bfloat16), b, c, sa, sb)
     with pytest.raises(RuntimeError, match="scales must be"):
         tb.matmul_fp4(a, b, c, sa.T.contiguous(), sb)
+
+
+def _streamk_ranges(total, G, units, cut):
+    """The K ranges the kernels give their workgroups for `cut` tiles at the end of a table (units of K per tile):
+    workgroup i takes q units, the first `rem` workgroups one more, in the order of their ids."""
+    first = (total - cut) * units
+    q, rem = divmod(cut * units, G)
+    return [(first + i * q + min(i, rem), first + (i + 1) * q + min(i + 1, rem)) for i in range(G)]
+
+
+@pytest.mark.parametrize("G", [1, 5, 8, 12, 256])
+def test_streamk_tail_rule_by_brute_force(G):
+    """tb_streamk_tail_tiles against a walk of the ranges it implies: the answer is 0, the tail or the tail plus one
+    round; the ranges cover every K unit of the cut tiles exactly once; no tile meets more ranges than the rule charged
+    for; and among the three plans the answer is the cheapest by the critical path of that walk (whole rounds, then the
+    longest range, then one exchange per extra piece of the most-cut tile)."""
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(G)
+    for _ in range(300):
+        total = int(rng.integers(1, 6 * G + 2))
+        units = int(rng.integers(1, 17))
+        unit_steps = int(rng.choice([1, 4]))
+        fix = int(rng.integers(0, 40))
+        cut = lib.tb_streamk_tail_tiles(total, G, units, unit_steps, fix)
+        tail, rounds = total % G, total // G
+        assert cut in {0, tail, tail + G} and cut <= total
+        if tail == 0 or units < 2:
+            assert cut == 0
+            continue
+
+        def walk_cost(c):
+            if c == 0:
+                return (rounds + 1) * units * unit_steps
+            ranges = _streamk_ranges(total, G, units, c)
+            cover = np.zeros(total * units, dtype=np.int32)
+            pieces = {}
+            for lo, hi in ranges:
+                cover[lo:hi] += 1
+                for t in range(lo // units, (hi + units - 1) // units if hi > lo else lo // units):
+                    pieces[t] = pieces.get(t, 0) + 1
+            assert (cover[(total - c) * units:] == 1).all() and (cover[:(total - c) * units] == 0).all()
+            longest = max(hi - lo for lo, hi in ranges)
+            return ((total - c) // G) * units * unit_steps + longest * unit_steps, max(pieces.values())
+
+        options = [0, tail] + ([tail + G] if rounds >= 1 else [])
+        costs = {}
+        for c in options:
+            if c == 0:
+                costs[c] = walk_cost(0)
+            else:
+                base, most = walk_cost(c)
+                # the rule's bound on the pieces of a tile is an upper bound of what the walk shows, and tight enough
+                # that both agree on the price within one exchange
+                q = (c * units) // G
+                bound = min(units, ((units - 2) // max(q, 1) if units >= 2 else 0) + 2)
+                assert most <= bound, (total, G, units, c, most, bound)
+                costs[c] = base + (bound - 1) * fix
+        assert costs[cut] == min(costs.values()), (total, G, units, unit_steps, fix, cut, costs)
+
+
+def test_streamk_tail_rule_known_answers():
+    """8 experts' 2072 tiles of 32 K steps on 256 workgroups: 8 whole rounds and 24 tiles.  Cutting the 24 tiles alone
+    means eight pieces per tile; cutting them together with one whole round means two: with exchanges at 9 K steps the
+    rule takes 280, at the library's 64 K steps it leaves the tiles whole, and with four times the K it cuts again."""
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    assert lib.tb_streamk_tail_tiles(2072, 256, 8, 4, 9) == 280
+    assert lib.tb_streamk_tail_tiles(2072, 256, 8, 4, 64) == 0
+    assert lib.tb_streamk_tail_tiles(2072, 256, 32, 4, 64) == 280
+    assert lib.tb_streamk_tail_tiles(2048, 256, 8, 4, 9) == 0          # whole rounds only
+    assert lib.tb_streamk_tail_tiles(256 + 200, 256, 8, 4, 9) == 0     # a nearly full last round is cheaper whole
+    assert lib.tb_streamk_tail_tiles(256 + 128, 256, 8, 4, 0) == 128   # free exchanges: always cut
+    assert lib.tb_streamk_tail_tiles(100, 256, 8, 4, 9) in (0, 100)
+    assert lib.tb_streamk_tail_tiles(10, 0, 8, 4, 9) == -10 and lib.tb_streamk_tail_tiles(10, 4, 8, 0, 9) == -10

@@ -25,7 +25,7 @@ TB_WS_QUEUES, TB_WS_GLOBAL_ATOMIC, TB_WS_HIERARCHICAL = 0, 1, 2
 
 EXPORTED_SYMBOLS = [
     "tb_abi_version", "tb_status_string", "tb_device_info", "tb_select", "tb_list_tiles", "tb_gemm",
-    "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_hadamard_mxfp4_quant",
+    "tb_workspace_bytes", "tb_gemm_fp4", "tb_grouped_gemm_fp8", "tb_grouped_workspace_bytes", "tb_streamk_tail_tiles", "tb_hadamard_mxfp4_quant",
     "tb_tile_coords", "tb_default_panel", "tb_ws_queue_tile", "tb_hierarchical_split",
     "tb_workspace_layout", "tb_debug_option", "tb_gemm_static_workspace", "tb_static_workspace_status", "tb_gemm_launch_info",
 ]
@@ -88,7 +88,8 @@ class tb_grouped_gemm_desc(C.Structure):
                 ("c_stride_m", C.c_int64), ("c_stride_n", C.c_int64), ("a_scale", C.c_void_p),
                 ("w_scale", C.c_void_p), ("group_offsets", C.c_void_p), ("block_m", C.c_int32),
                 ("block_n", C.c_int32), ("block_k", C.c_int32), ("group_m", C.c_int32), ("num_xcds", C.c_int32),
-                ("small_rows", C.c_int32)]
+                ("small_rows", C.c_int32), ("streamk", C.c_int32), ("epoch", C.c_uint32), ("spin_limit", C.c_uint32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
 class tb_quant_desc(C.Structure):
@@ -122,6 +123,9 @@ def load():
     lib.tb_workspace_bytes.restype = C.c_size_t
     lib.tb_gemm_fp4.argtypes = [C.POINTER(tb_gemm_fp4_desc), C.c_void_p]
     lib.tb_grouped_gemm_fp8.argtypes = [C.POINTER(tb_grouped_gemm_desc), C.c_void_p]
+    lib.tb_grouped_workspace_bytes.argtypes = [C.POINTER(tb_grouped_gemm_desc)]
+    lib.tb_grouped_workspace_bytes.restype = C.c_size_t
+    lib.tb_streamk_tail_tiles.argtypes = [C.c_int32] * 5
     lib.tb_hadamard_mxfp4_quant.argtypes = [C.POINTER(tb_quant_desc), C.c_void_p]
     lib.tb_tile_coords.argtypes = [C.c_int32] * 5 + [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     lib.tb_default_panel.argtypes = [C.c_int32] * 3

@@ -95,6 +95,10 @@ struct GemmParams {
   int32_t grp_phase, grp_big, grp_thr;
   int32_t grp_auto, grp_small_bm;
   int32_t grp_other_tn, grp_other_grid;   // column tiles and grid of the other launch
+  // grouped with a Stream-K tail (4-wave kernels): the tiles that do not fill whole rounds of the grid are cut into
+  // K ranges as in MODE_SK; how many that is follows from the row counts, so every workgroup works it out
+  // itself (sk_tail_tiles).  grp_sk_fix: what one extra piece of a tile costs its owner, in K steps.
+  int32_t grp_sk, grp_sk_fix;
 };
 
 struct TileCtx {
@@ -1106,6 +1110,18 @@ __device__ __forceinline__ void partial_add(const float* slot, v4f (&acc)[T::TM]
 #endif
 }
 
+// A value every lane holds alike, as a scalar register (an "s" operand of an assembly statement must
+// be one; the compiler does not move a value it keeps in a vector register there by itself).
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ uint32_t uniform(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ const float* uniform(const float* p) { return (const float*)uniform((const uint8_t*)p); }
+
 // ------------------------------------------------------------------------------------------------
 // work items: which (tile, k range) a workgroup runs next, for each schedule
 // ------------------------------------------------------------------------------------------------
@@ -1146,18 +1162,26 @@ __device__ __forceinline__ int grouped_phase(const GemmParams& p, int grid) {
   return split ? 2 : -1;
 }
 
+// the row blocks of expert e in the table of a phase: their number, the first row and the row limit
+__device__ __forceinline__ int grouped_rows(const GemmParams& p, int phase, int e, int BM, int& base, int& lim) {
+  const int lo = p.group_offsets[e], hi = p.group_offsets[e + 1];
+  const int rows = max(hi - lo, 0);
+  int mb = (rows + BM - 1) / BM;
+  base = lo; lim = hi;
+  if (phase != 0) {
+    const int full = rows / p.grp_big, rem = rows - full * p.grp_big;
+    const bool small = rem > 0 && rem <= p.grp_thr;
+    if (phase == 1) { mb = full + ((rem > 0 && !small) ? 1 : 0); if (small) lim = lo + full * p.grp_big; }
+    else { mb = small ? (rem + BM - 1) / BM : 0; base = lo + full * p.grp_big; }
+  }
+  return mb;
+}
+
 __device__ __forceinline__ bool grouped_tile(const GemmParams& p, int phase, int tile, int BM, int BN, int USZ, TileCtx& tc) {
   int acc = 0;
   for (int e = 0; e < p.num_groups; ++e) {
-    const int lo = p.group_offsets[e], hi = p.group_offsets[e + 1];
-    const int rows = max(hi - lo, 0);
-    int mb = (rows + BM - 1) / BM, base = lo, lim = hi;
-    if (phase != 0) {
-      const int full = rows / p.grp_big, rem = rows - full * p.grp_big;
-      const bool small = rem > 0 && rem <= p.grp_thr;
-      if (phase == 1) { mb = full + ((rem > 0 && !small) ? 1 : 0); if (small) lim = lo + full * p.grp_big; }
-      else { mb = small ? (rem + BM - 1) / BM : 0; base = lo + full * p.grp_big; }
-    }
+    int base, lim;
+    const int mb = grouped_rows(p, phase, e, BM, base, lim);
     const int cnt = mb * p.tiles_n;
     if (tile < acc + cnt) {
       const int local = tile - acc;
@@ -1173,6 +1197,45 @@ __device__ __forceinline__ bool grouped_tile(const GemmParams& p, int phase, int
   return false;
 }
 
+__device__ __forceinline__ int grouped_total(const GemmParams& p, int phase, int BM) {
+  int acc = 0;
+  for (int e = 0; e < p.num_groups; ++e) {
+    int base, lim;
+    acc += grouped_rows(p, phase, e, BM, base, lim) * p.tiles_n;
+  }
+  return acc;
+}
+
+// A table of `total` tiles of `units` K units each (a unit = `unit_steps` K steps) on a resident grid of G
+// workgroups: how many tiles at the table's end are cut into K ranges, one range per workgroup, instead of
+// running as whole tiles.  Three plans are priced in K steps for the critical path of a workgroup: whole tiles
+// only (one more round, however few tiles it holds); the tiles past the last whole round shared out; those and
+// one whole round shared out (every range then covers more than a tile, so no tile has more than two pieces).
+// A tile cut into n pieces costs its owner (n - 1) * fix_steps: the partial sums go through memory.
+__host__ __device__ inline int sk_tail_pieces(int units, int range) {
+  // the most ranges of `range` units a tile of `units` units can meet
+  if (range < 1) range = 1;
+  const int n = (units >= 2 ? (units - 2) / range : 0) + 2;
+  return n < units ? n : units;
+}
+__host__ __device__ inline int sk_tail_tiles(int total, int G, int units, int unit_steps, int fix_steps) {
+  if (total <= 0 || G <= 0 || units < 2) return 0;
+  const int tail = total % G, rounds = total / G;
+  if (tail == 0) return 0;
+  long long best = (long long)(rounds + 1) * units * unit_steps;
+  int pick = 0;
+  for (int extra = 0; extra <= 1; ++extra) {
+    if (extra > rounds) break;
+    const long long skt = tail + (long long)extra * G;
+    const long long all = skt * units;
+    const int range = (int)(all / G);
+    const long long cost = (long long)(rounds - extra) * units * unit_steps + ((all + G - 1) / G) * unit_steps +
+                           (long long)(sk_tail_pieces(units, range) - 1) * fix_steps;
+    if (cost < best) { best = cost; pick = (int)skt; }
+  }
+  return pick;
+}
+
 template <class T, bool SK>
 struct Sched {
   int pid, G;
@@ -1182,11 +1245,13 @@ struct Sched {
   int64_t start, last, q, rem;  // Stream-K iteration range of this workgroup
   int dp_tiles;
   int gphase;             // grouped: which tile table this launch runs
+  int gtotal;             // grouped with a Stream-K tail: entries of that table
   bool ws_phase;          // Stream-K with work stealing: still drawing whole tiles from the queues
 
   __device__ __forceinline__ void init(const GemmParams& p) {
     G = gridDim.x;
     gphase = p.mode == MODE_GROUPED ? grouped_phase(p, G) : 0;
+    gtotal = 0;
     pid = blockIdx.x;
     sk_id = blockIdx.x;
     if (p.mode != MODE_WS && p.num_xcds > 1) pid = chiplet_transform_chunked(pid, G, p.num_xcds, p.chunk);
@@ -1206,6 +1271,20 @@ struct Sched {
       const int64_t ipt = p.k_iters / max(1, p.sk_unit);
       start = (int64_t)dp_tiles * ipt + sk_id * q + min((int64_t)sk_id, rem);
       last = (int64_t)dp_tiles * ipt + (sk_id + 1) * q + min((int64_t)sk_id + 1, rem);
+    }
+    if constexpr (SK) {
+      if (p.mode == MODE_GROUPED && p.grp_sk && gphase >= 0) {
+        // the table's real length is only known here; whole rounds first, the rest in K ranges (ordered as in MODE_SK)
+        const int unit = max(1, p.sk_unit);
+        const int64_t ipt = p.k_iters / unit;
+        gtotal = grouped_total(p, gphase, T::BM);
+        const int skt = sk_tail_tiles(gtotal, G, (int)ipt, unit, p.grp_sk_fix);
+        dp_tiles = gtotal - skt;
+        const int64_t total_sk = (int64_t)skt * ipt;
+        q = total_sk / G; rem = total_sk % G;
+        start = (int64_t)dp_tiles * ipt + sk_id * q + min((int64_t)sk_id, rem);
+        last = (int64_t)dp_tiles * ipt + (sk_id + 1) * q + min((int64_t)sk_id + 1, rem);
+      }
     }
     if (p.mode == MODE_WS && p.cu_mask && p.cu_mask[pid] == 0) step = 1 << 30;  // masked out: nothing to do
   }
@@ -1250,7 +1329,18 @@ struct Sched {
       return true;
   }
 
+  // The next work item.  Every lane computes the same one, partly from values read from memory (row offsets of a
+  // grouped launch, queue counters), which the compiler may keep in vector registers; what the K loops hand to
+  // assembly statements as scalar operands derives from these fields, so they are made scalars here.
   __device__ __forceinline__ bool next(const GemmParams& p, Work& w, int* s_bcast, int tid) {
+    const bool ok = next_item(p, w, s_bcast, tid);
+    w.tc.m0 = uniform(w.tc.m0); w.tc.n0 = uniform(w.tc.n0); w.tc.m_lim = uniform(w.tc.m_lim); w.tc.n_lim = uniform(w.tc.n_lim);
+    w.tc.B = uniform(w.tc.B); w.tc.sb = uniform(w.tc.sb);
+    w.it0 = uniform(w.it0); w.it1 = uniform(w.it1); w.kind = uniform(w.kind);
+    return ok;
+  }
+
+  __device__ __forceinline__ bool next_item(const GemmParams& p, Work& w, int* s_bcast, int tid) {
     w.it0 = 0; w.it1 = p.k_iters; w.kind = WK_FULL; w.seg_begin = w.tile_first = 0;
     if (p.mode == MODE_STATIC) {
       if (next_tile >= p.total_tiles) return false;
@@ -1261,10 +1351,20 @@ struct Sched {
     if (p.mode == MODE_GROUPED) {
       // the grid loops over the tile table; the first id past the table's end finishes the workgroup
       // (the host only knows an upper bound of the table's length)
-      if (gphase < 0 || next_tile >= p.total_tiles) return false;
-      bool ok = grouped_tile(p, gphase, next_tile, T::BM, T::BN, T::USZ, w.tc);
-      next_tile = ok ? next_tile + G : p.total_tiles;
-      return ok;
+      bool tail = false;
+      if constexpr (SK) tail = p.grp_sk != 0;
+      if (!tail) {
+        if (gphase < 0 || next_tile >= p.total_tiles) return false;
+        bool ok = grouped_tile(p, gphase, next_tile, T::BM, T::BN, T::USZ, w.tc);
+        next_tile = ok ? next_tile + G : p.total_tiles;
+        return ok;
+      }
+      if (gphase < 0) return false;
+      if (next_tile < dp_tiles) {
+        grouped_tile(p, gphase, next_tile, T::BM, T::BN, T::USZ, w.tc);
+        next_tile += G;
+        return true;
+      }
     }
     if (p.mode == MODE_WS) {
       // Queues: one counter per (xcd, slot).  A workgroup drains its own queue, then the other
@@ -1315,9 +1415,12 @@ struct Sched {
       return queue_next(p, p.total_tiles, pid, w, s_bcast, tid);
     }
     if constexpr (!SK) return false;
+    const bool grouped = p.mode == MODE_GROUPED;
     // MODE_SK: data-parallel tiles first (from the work-stealing queues when asked for, reference
     // kernels/streamk_gemm_work_stealing.py:9-418), then this workgroup's share of the Stream-K iterations
-    if (ws_phase) {
+    if (grouped) {
+      // (its whole tiles were handed out above)
+    } else if (ws_phase) {
       if (queue_next(p, dp_tiles, sk_id, w, s_bcast, tid)) return true;
       ws_phase = false;
       step = 0;
@@ -1336,7 +1439,8 @@ struct Sched {
     const int64_t tile_first = (int64_t)tile * ipt;
     const int64_t tile_end = tile_first + ipt;
     const int64_t begin = max(tile_first, start);
-    plain_tile(p, tile, T::BM, T::BN, w.tc);
+    if (grouped) grouped_tile(p, gphase, tile, T::BM, T::BN, T::USZ, w.tc);
+    else plain_tile(p, tile, T::BM, T::BN, w.tc);
     w.it0 = (int)(begin - tile_first) * unit;
     w.it1 = (int)(last - tile_first) * unit;
     w.kind = (last != tile_end) ? WK_SK_PUBLISH : WK_SK_OWNER;
@@ -1349,7 +1453,7 @@ struct Sched {
 // What the last workgroup of a Stream-K launch to leave does: advance the launch count the workspace keeps (every
 // workgroup has read it before it gets here) and rearm the work-stealing queues if the launch drew from them.
 __device__ __forceinline__ void sk_leave(const GemmParams& p, uint32_t epoch, int tid) {
-  if (p.mode != MODE_SK || tid != 0 || (p.epoch != EPOCH_ON_DEVICE && !p.sk_ws)) return;
+  if (!(p.mode == MODE_SK || (p.mode == MODE_GROUPED && p.grp_sk)) || tid != 0 || (p.epoch != EPOCH_ON_DEVICE && !p.sk_ws)) return;
   const uint32_t done = atomicAdd(p.ctl + CTL_DONE, 1u);
   if (done != gridDim.x - 1) return;
   if (p.sk_ws)

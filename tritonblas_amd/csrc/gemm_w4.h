@@ -36,17 +36,6 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// A value every lane holds alike, as a scalar register (an "s" operand of an assembly statement must
-// be one; the compiler does not move a value it keeps in a vector register there by itself).
-__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
-__device__ __forceinline__ uint32_t uniform(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
-__device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
-  const uint64_t v = (uint64_t)(uintptr_t)p;
-  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
-  return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
-}
-
 // accumulator register a[N] (written by the K loop statement; the compiler never allocates these);
 // INT: the K loop left an int32 sum there
 template <int N, bool INT = false>

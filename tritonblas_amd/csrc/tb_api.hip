@@ -81,6 +81,7 @@ struct Hooks {
   int panel = -1;               // TB_PANEL=<n>: column panel width of the tile order (-1: the library's)
   int no_column_split = 0, force_column_split = 0;
   int quant_div64 = 0;          // TB_QUANT_DIV64=1: the quantiser's kernel for 2^31 items and more at any size
+  int grp_sk_fix = 0;           // TB_GRP_SK_FIX=<K steps>: what the grouped Stream-K tail's model charges per extra piece of a tile
   int lab = 0;                  // TB_DEBUG=<bits>: 4 = the 4-wave kernels store every tile with their compiled epilogue (none fused
                                 // into the next K loop); 1, 2 = only acted on by kernels built with TB_LAB_HOOKS
 };
@@ -105,6 +106,7 @@ void read_hooks() {
   g_hooks.force_column_split = env_int("TB_FORCE_COLUMN_SPLIT", 0);
   g_hooks.quant_div64 = env_int("TB_QUANT_DIV64", 0);
   g_hooks.lab = env_int("TB_DEBUG", 0);
+  g_hooks.grp_sk_fix = env_int("TB_GRP_SK_FIX", 0);
 }
 std::mutex g_hooks_mu;
 // (a copy taken under the hooks' own lock: tb_debug_option may change one while another thread plans)
@@ -208,6 +210,7 @@ struct Job {
   const int32_t* group_offsets = nullptr; int num_groups = 0;
   int64_t b_group_stride = 0, sb_group_stride = 0;
   int grp_phase = 0, grp_big = 0, grp_thr = 0, grp_auto = 0;   // see GemmParams
+  int grp_sk = 0;          // grouped: cut the tiles that do not fill whole rounds of the grid into K ranges (needs a workspace)
   int column_split = 0;
 };
 
@@ -389,6 +392,20 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     p.total_tiles = (int32_t)bound;
     grid = (int)std::min<int64_t>(bound, resident);
     if (hooks().grid > 0) grid = (int)std::min<int64_t>(bound, hooks().grid);
+    // Stream-K tail: only the hand-scheduled 4-wave kernel has the cheap exchange of partial tiles that makes
+    // it pay (K ranges in blocks of four steps), and only the launch of the tall tiles
+    if (j.grp_sk && p.grp_phase != 2 && v->k_step_pairs && v->kernel_sk && p.k_iters % 4 == 0 && p.k_iters >= 8 && occ == 1) {
+      p.grp_sk = 1;
+      // (measured with 8 experts, 2072 tiles of 32 K steps on 256 workgroups: the launch that cuts 280 tiles
+      // takes 63 us longer than 7 whole rounds and 35 K steps would -- every workgroup writes and reads a
+      // 256 KB partial tile while the operand strips already keep the fabric busy -- i.e. about 48 K steps, and
+      // the kernel that can cut is 12 us slower than the one that cannot even when it cuts nothing)
+      p.grp_sk_fix = hooks().grp_sk_fix > 0 ? hooks().grp_sk_fix : 64;
+      p.sk_unit = 4;
+      plan->ws_flags_off = WS_FLAGS_OFF;
+      plan->ws_p_off = plan->ws_flags_off + (((size_t)grid * 4 + 255) / 256) * 256;
+      plan->ws_need = plan->ws_p_off + (size_t)grid * v->bm * v->bn * 4;
+    }
   } else if (j.schedule == TB_SCHED_PERSISTENT) {
     // a resident grid that loops over the tiles (matmul.py:160-198: for tile_id in range(pid, total, NUM_SMS))
     p.mode = MODE_STATIC;
@@ -505,7 +522,7 @@ PlanKey plan_key(const Job& j, int dev) {
       j.dt, j.c_type, j.bias_type, j.schedule, dev, j.M, j.N, j.K, j.a_sr, j.a_sk, j.b_sr, j.b_sk, j.c_sm, j.c_sn,
       j.mxa_sr, j.mxa_sk, j.mxb_sr, j.mxb_sk, j.bias_stride, j.bm, j.bn, j.bk, j.group_m, j.num_xcds, j.grid,
       j.counters_per_xcd, j.ws_mode, j.ws_local, j.cu_mask_len, j.ws_global, j.num_groups, j.grp_phase, j.grp_big,
-      j.grp_thr, j.grp_auto, j.b_group_stride, j.sb_group_stride, al(j.A), al(j.B), al(j.C), al(j.mxa), al(j.mxb),
+      j.grp_thr, j.grp_auto, j.grp_sk, j.b_group_stride, j.sb_group_stride, al(j.A), al(j.B), al(j.C), al(j.mxa), al(j.mxb),
       al(j.bias), j.sa ? 1 : 0, j.sb ? 1 : 0, j.cu_mask ? 1 : 0, j.group_offsets ? 1 : 0, j.column_split,
       (int64_t)g_hooks_version};
   static_assert(sizeof(f) <= sizeof(k.v), "PlanKey too small");
@@ -574,14 +591,14 @@ int run_plan(const Job& j, Plan& plan, hipStream_t stream) {
     if (!j.workspace || j.workspace_bytes < plan.ws_need || ((uintptr_t)j.workspace & 255)) return TB_ERR_WORKSPACE;
     // Stream-K flags carry the launch epoch and are never cleared: epoch 0 is what a fresh, zeroed
     // workspace holds in every flag, so a launch tagged 0 would take unpublished partial tiles for published
-    if (p.mode == MODE_SK && j.epoch == 0) return TB_ERR_BAD_ARGUMENT;
+    if ((p.mode == MODE_SK || p.grp_sk) && j.epoch == 0) return TB_ERR_BAD_ARGUMENT;
     uint8_t* ws = (uint8_t*)j.workspace;
     p.ctl = (uint32_t*)ws;
     if (p.mode == MODE_WS || p.sk_ws) p.counters = (int32_t*)(ws + plan.ws_counters_off);
-    if (p.mode == MODE_SK) { p.flags = (uint32_t*)(ws + plan.ws_flags_off); p.P = (float*)(ws + plan.ws_p_off); }
+    if (p.mode == MODE_SK || p.grp_sk) { p.flags = (uint32_t*)(ws + plan.ws_flags_off); p.P = (float*)(ws + plan.ws_p_off); }
   }
   void* args[] = {(void*)&p};
-  const void* kern = (p.mode == MODE_SK) ? plan.v->kernel_sk : plan.v->kernel;
+  const void* kern = (p.mode == MODE_SK || p.grp_sk) ? plan.v->kernel_sk : plan.v->kernel;
   hipError_t e = hipLaunchKernel(kern, dim3((unsigned)plan.grid), dim3((unsigned)plan.v->threads), args, 0, stream);
   if (e != hipSuccess) { (void)hipGetLastError(); return TB_ERR_LAUNCH; }
   return TB_OK;
@@ -768,7 +785,8 @@ int tb_debug_option(const char* name, int value) {
   struct { const char* n; int* p; } table[] = {
       {"waves", &g_hooks.waves}, {"no_mxlds", &g_hooks.no_mxlds}, {"no_cline", &g_hooks.no_cline},
       {"no_skinny", &g_hooks.no_skinny}, {"skinny", &g_hooks.skinny}, {"grid", &g_hooks.grid}, {"panel", &g_hooks.panel},
-      {"no_column_split", &g_hooks.no_column_split}, {"force_column_split", &g_hooks.force_column_split}, {"quant_div64", &g_hooks.quant_div64}, {"lab", &g_hooks.lab}};
+      {"no_column_split", &g_hooks.no_column_split}, {"force_column_split", &g_hooks.force_column_split}, {"quant_div64", &g_hooks.quant_div64}, {"lab", &g_hooks.lab},
+      {"grp_sk_fix", &g_hooks.grp_sk_fix}};
   for (auto& t : table)
     if (std::strcmp(t.n, name) == 0) { *t.p = value; ++g_hooks_version; return TB_OK; }
   return TB_ERR_BAD_ARGUMENT;
@@ -932,10 +950,10 @@ int tb_gemm_fp4(const tb_gemm_fp4_desc* d, void* stream) {
 // the short FP8 tile the second launch of a grouped GEMM runs
 constexpr int kGroupedSmallBM = 32, kGroupedSmallBN = 128, kGroupedSmallBK = 256;
 
-int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
+// the job of the (first) launch; *two: a second launch with the short tile may follow
+static int job_from_grouped(const tb_grouped_gemm_desc* d, Job* out, bool* two) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_grouped_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
-  if (!d->a || !d->w || !d->c || !d->group_offsets) return TB_ERR_NULL_POINTER;
   if ((d->a_scale == nullptr) != (d->w_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
   if (d->num_groups <= 0) return TB_ERR_BAD_SHAPE;
   Job j;
@@ -949,17 +967,52 @@ int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
   j.group_offsets = d->group_offsets; j.num_groups = d->num_groups;
   j.b_group_stride = d->w_stride_g; j.sb_group_stride = d->n;
   if ((d->w_stride_g * 1) % 16) return TB_ERR_BAD_LAYOUT;
+  if (d->streamk < 0 || d->streamk > 1) return TB_ERR_BAD_ARGUMENT;
+  if (d->streamk) {
+    j.grp_sk = 1;
+    j.workspace = d->workspace; j.workspace_bytes = d->workspace_bytes;
+    j.epoch = d->epoch; j.spin_limit = d->spin_limit;
+  }
   // Two launches unless switched off or a tile is forced: tall tiles for whole row blocks and long
   // remainders, then a short streaming tile for the experts whose last block holds few rows (the row
   // counts live on the device, so both tile tables are evaluated there; an empty second table costs
   // one empty launch).
   if (d->small_rows < -1) return TB_ERR_BAD_ARGUMENT;
   const int thr = d->small_rows > 0 ? d->small_rows : 64;
-  const bool two = d->small_rows > 0 || (d->small_rows == 0 && d->block_m == 0);
-  if (!two || d->k % kGroupedSmallBK) return launch(j, (hipStream_t)stream);
-  j.grp_phase = 1; j.grp_thr = thr; j.grp_auto = d->small_rows == 0;
+  *two = (d->small_rows > 0 || (d->small_rows == 0 && d->block_m == 0)) && d->k % kGroupedSmallBK == 0;
+  if (*two) { j.grp_phase = 1; j.grp_thr = thr; j.grp_auto = d->small_rows == 0; }
+  *out = j;
+  return TB_OK;
+}
+
+size_t tb_grouped_workspace_bytes(const tb_grouped_gemm_desc* d) {
+  Job j;
+  bool two = false;
+  if (job_from_grouped(d, &j, &two) != TB_OK || !j.grp_sk) return 0;
   tb_hw hw;
-  int st = current_hw(&hw);
+  bool have_dev = current_hw(&hw) == TB_OK;
+  if (!have_dev) default_hw(&hw);
+  Plan plan;
+  if (make_plan(j, hw, have_dev, &plan) != TB_OK) return 0;
+  return plan.ws_need;
+}
+
+int tb_streamk_tail_tiles(int32_t total_tiles, int32_t grid, int32_t k_units, int32_t unit_steps, int32_t fix_steps) {
+  if (total_tiles < 0 || grid <= 0 || k_units <= 0 || unit_steps <= 0 || fix_steps < 0) return TB_ERR_BAD_ARGUMENT;
+  return sk_tail_tiles(total_tiles, grid, k_units, unit_steps, fix_steps);
+}
+
+int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
+  if (!d) return TB_ERR_NULL_POINTER;
+  if (d->struct_bytes != sizeof(tb_grouped_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
+  if (!d->a || !d->w || !d->c || !d->group_offsets) return TB_ERR_NULL_POINTER;
+  Job j;
+  bool two = false;
+  int st = job_from_grouped(d, &j, &two);
+  if (st != TB_OK) return st;
+  if (!two) return launch(j, (hipStream_t)stream);
+  tb_hw hw;
+  st = current_hw(&hw);
   if (st != TB_OK) return st;
   Plan first, second;
   st = cached_plan(j, hw, &first);
@@ -968,6 +1021,7 @@ int tb_grouped_gemm_fp8(const tb_grouped_gemm_desc* d, void* stream) {
   Job j2 = j;
   j2.bm = kGroupedSmallBM; j2.bn = kGroupedSmallBN; j2.bk = kGroupedSmallBK;
   j2.grp_phase = 2; j2.grp_big = first.p.grp_big;
+  j2.grp_sk = 0; j2.workspace = nullptr; j2.workspace_bytes = 0;
   st = cached_plan(j2, hw, &second);
   if (st != TB_OK) return st;
   first.p.grp_small_bm = second.p.grp_small_bm = second.v->bm;

@@ -415,12 +415,19 @@ def matmul_fp4(a, b, c, a_scales, b_scales, block_m: int = None, block_n: int = 
 
 
 def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int = None, block_n: int = None,
-                        block_k: int = None, small_rows: int = 0):
+                        block_k: int = None, small_rows: int = 0, enable_streamk: bool = False,
+                        config: MatmulConfig = None):
     """Grouped (MoE) FP8 GEMM: rows ``group_offsets[e]:group_offsets[e+1]`` of ``a`` (M, K) meet expert
     weight ``w[e]`` (N, K); ``c[rows] = cast((a[rows] @ w[e].T) * a_scale[rows, None] * w_scale[e][None, :])``.
     ``group_offsets`` is an int32 device tensor of E+1 ascending row offsets.  No host sync: the row counts
     are only read on the device.  An expert's last partial row block of at most ``small_rows`` rows goes to a
-    second launch with a 32-row tile (0: the library's default of 64 rows, off when a tile is forced; -1: off)."""
+    second launch with a 32-row tile (0: the library's default of 64 rows, off when a tile is forced; -1: off).
+    ``enable_streamk``: the tiles that do not fill whole rounds of the launch grid are cut into K ranges when the
+    row counts make that cheaper than one more round (decided on the device; only those tiles' summation order
+    changes).  The flags and partial tiles live in ``config``'s workspace, by default the one this package keeps
+    per device and stream.  Off by default: exchanging 256x256 partial tiles costs about as much as 50 K steps, so it
+    only pays for long K (beyond about 8192 for FP8), and the kernel that can cut tiles is 2-3 % slower when it
+    does not."""
     M, K = a.shape
     E, N, K2 = w.shape
     assert K == K2 and c.shape[0] == M and c.shape[1] == N, "Incompatible Dimensions"
@@ -449,5 +456,16 @@ def grouped_matmul_a8w8(a, w, a_scale, w_scale, c, group_offsets, block_m: int =
         d.block_m, d.block_n, d.block_k = block_m, block_n, block_k
     d.small_rows = small_rows
     with _on_device(dev):
-        _lib.check(_lib.load().tb_grouped_gemm_fp8(d, _lib.stream_handle(dev)), "tb_grouped_gemm_fp8")
+        lib = _lib.load()
+        if enable_streamk:
+            d.streamk = 1
+            need = lib.tb_grouped_workspace_bytes(d)
+            if need:
+                cfg = config if config is not None else _stream_config(dev)
+                ws = cfg.ensure(need)
+                d.workspace, d.workspace_bytes = ws.data_ptr(), ws.numel()
+                d.epoch, d.spin_limit = _lib.TB_EPOCH_ON_DEVICE, cfg.spin_limit
+            else:
+                d.streamk = 0
+        _lib.check(lib.tb_grouped_gemm_fp8(d, _lib.stream_handle(dev)), "tb_grouped_gemm_fp8")
     return c
