@@ -47,9 +47,9 @@ enum {
   TB_FP8_E5M2 = 6   /* OCP e5m2, operands of tb_gemm only (the type utils.py:46 lists next to e4m3); both
                        operands must have the same 8-bit format                                     */
 };
-/* TB_FP8_E4M3 is also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 or TB_FP8_E5M2 operands: the fp32 epilogue
- * result is clamped to +-448 and rounded to nearest even (the reference's a8w8 oracle,
- * tests/test_matmul_a8w8_lt.py:11-38). */
+/* TB_FP8_E4M3 and TB_FP8_E5M2 are also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 or TB_FP8_E5M2 operands:
+ * the fp32 epilogue result is clamped to the format's largest finite value (+-448, +-57344; NaN stays NaN) and rounded
+ * to nearest even (the reference's a8w8 oracle, tests/test_matmul_a8w8_lt.py:11-38). */
 
 /* ---- schedules ------------------------------------------------------------------------------ */
 enum {

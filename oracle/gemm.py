@@ -74,7 +74,7 @@ def ref_gemm(a: torch.Tensor, b: torch.Tensor, out_dtype=None, a_scale=None, b_s
         acc = acc + bias.to(torch.float32)[None, :]
     if out_dtype is None:
         out_dtype = a.dtype
-    if out_dtype in (torch.float8_e4m3fn,):
+    if out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2):   # tests/test_matmul_a8w8_lt.py:27-32
         mx = torch.finfo(out_dtype).max
         acc = torch.clamp(acc, -mx, mx)
     return acc.to(out_dtype)

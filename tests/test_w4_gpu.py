@@ -444,45 +444,53 @@ def test_a8w8_fp8_output_keeps_nan():
         torch.testing.assert_close(got[fin], want[fin], atol=2.0, rtol=0.2)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
 @pytest.mark.parametrize("m,n,k", [(512, 768, 512), (300, 500, 768), (1, 257, 512), (2048, 1280, 1024)])
-def test_fp8_four_wave_kernel_e4m3_output(m, n, k, tb_option):
-    """e4m3 results straight from the 4-wave kernel's accumulators (eight bytes per lane and row block): the same
-    bytes as the 8-wave kernel's, NaN kept, the reference's tolerance against the oracle."""
+def test_fp8_four_wave_kernel_e4m3_output(m, n, k, out_dtype, tb_option):
+    """8-bit float results (e4m3, e5m2) straight from the 4-wave kernel's accumulators (eight bytes per lane and row
+    block): the same bytes as the 8-wave kernel's, NaN kept, the reference's tolerance against the oracle (for e5m2
+    widened to one unit in its last place, 25 %)."""
     aq, bq, sa, sb = _fp8_case(m, n, k, 93)
-    sa = sa * 40.0
+    sa = sa * (40.0 if out_dtype == torch.float8_e4m3fn else 5000.0)   # part of the result beyond the format's range
     sa[0] = float("nan")
     outs = {}
     for waves in (22, 24):
-        outs[waves] = _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=torch.float8_e4m3fn)
-    want = OG.ref_gemm(aq, bq, torch.float8_e4m3fn, a_scale=sa, b_scale=sb)
+        outs[waves] = _run_fp8(aq, bq, sa, sb, waves, tb_option, out_dtype=out_dtype)
+    want = OG.ref_gemm(aq, bq, out_dtype, a_scale=sa, b_scale=sb)
     assert torch.equal(outs[22].view(torch.uint8), outs[24].view(torch.uint8))
     got = outs[22].float()
     assert torch.isnan(got[0]).all() and not torch.isnan(got[1:]).any()
-    torch.testing.assert_close(got[1:], want.float()[1:], atol=2.0, rtol=0.2)
+    # (the e5m2 case scales its sums 125 times as far up, and the absolute tolerance with them)
+    e4 = out_dtype == torch.float8_e4m3fn
+    torch.testing.assert_close(got[1:], want.float()[1:], atol=2.0 if e4 else 250.0, rtol=0.2 if e4 else 0.26)
     if m > 1:
         same = (outs[22][1:].view(torch.uint8) == want[1:].view(torch.uint8)).float().mean().item()
         assert same >= 0.99
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 256), (100, 300, 640), (512, 1024, 512)])
 @pytest.mark.parametrize("streamk", [False, True])
-def test_a8w8_fp8_output(m, n, k, streamk):
-    """a8w8 with an e4m3 result: clamp to +-448, round to nearest even -- the reference's oracle and
-    tolerances for this case (tests/test_matmul_a8w8_lt.py:11-38, :108-112: atol 2.0, rtol 0.2)."""
+def test_a8w8_fp8_output(m, n, k, streamk, out_dtype):
+    """a8w8 with an 8-bit float result: clamp to the format's largest finite value (448, 57344), round to nearest even
+    -- the reference's oracle and tolerances for this case (tests/test_matmul_a8w8_lt.py:11-38, :108-112: atol 2.0,
+    rtol 0.2; e5m2, whose steps are 25 % and whose case is scaled 125 times as far up, at rtol 0.26 and atol 250)."""
     import tritonblas_amd as tb
     aq, bq, sa, sb = _fp8_case(m, n, k, 91)
-    sa = sa * 40.0   # push part of the result beyond the e4m3 range so that the clamp is exercised
+    e4 = out_dtype == torch.float8_e4m3fn
+    sa = sa * (40.0 if e4 else 5000.0)   # push part of the result beyond the format's range so that the clamp is exercised
     a, b = aq.cuda(), bq.T.contiguous().cuda().T
-    c = torch.zeros(m, n, dtype=torch.float8_e4m3fn, device="cuda")
+    c = torch.zeros(m, n, dtype=out_dtype, device="cuda")
     tb.matmul_a8w8(a, b, sa.cuda(), sb.cuda(), c, enable_streamk=streamk)
-    want = OG.ref_gemm(aq, bq, torch.float8_e4m3fn, a_scale=sa, b_scale=sb)
+    want = OG.ref_gemm(aq, bq, out_dtype, a_scale=sa, b_scale=sb)
     got = c.float().cpu()
-    assert not torch.isnan(got).any()
-    assert got.abs().max() <= 448.0
-    torch.testing.assert_close(got, want.float(), atol=2.0, rtol=0.2)
-    # the rounding itself: at most one e4m3 step away from the oracle's cast, and mostly identical
+    assert not torch.isnan(got).any() and not torch.isinf(got).any()
+    lim = 448.0 if e4 else 57344.0
+    assert got.abs().max() == lim, "the case is meant to reach the clamp"
+    torch.testing.assert_close(got, want.float(), atol=2.0 if e4 else 250.0, rtol=0.2 if e4 else 0.26)
+    # the rounding itself: at most one step away from the oracle's cast, and mostly identical
     same = (c.cpu().view(torch.uint8) == want.view(torch.uint8)).float().mean().item()
-    assert same >= 0.99, f"only {same:.4f} of the e4m3 codes match the oracle's"
+    assert same >= 0.99, f"only {same:.4f} of the codes match the oracle's"
 
 
 # ---- Stream-K on the 4-wave kernels, and Stream-K with work stealing ------------------------------------------

@@ -838,18 +838,32 @@ __device__ __forceinline__ float load_as_f32(const uint8_t* p, int type) {
   return __builtin_bit_cast(float, u);
 }
 
+// four fp32 values as four bytes of an 8-bit float format: clamped to its largest finite value (NaN kept), nearest even
+template <int CT>
+__device__ __forceinline__ int pack4_f8(float a, float b, float c, float d) {
+  constexpr float lim = CT == DT_FP8 ? 448.f : 57344.f;
+  float x[4] = {a, b, c, d};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) x[j] = (x[j] != x[j]) ? x[j] : fminf(fmaxf(x[j], -lim), lim);
+  int w;
+  if constexpr (CT == DT_FP8) {
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3], w, true);
+  } else {
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(x[0], x[1], 0, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(x[2], x[3], w, true);
+  }
+  return w;
+}
+
 template <int CT>
 __device__ __forceinline__ void store4(uint8_t* C, int64_t off_el, int64_t sn, v4f v, int nvalid, bool vec) {
-  if constexpr (CT == DT_FP8) {
-    // fp32 -> e4m3fn: clamp to the largest finite value, then round to nearest even
+  if constexpr (is_f8(CT)) {
+    // fp32 -> e4m3fn / e5m2: clamp to the largest finite value, then round to nearest even
     // (the reference's a8w8 oracle, tests/test_matmul_a8w8_lt.py:11-38).  torch.clamp keeps NaN, and so
     // does this: fmaxf / fminf return their other argument for a NaN, which would turn a poisoned or
-    // overflowed-to-NaN result into a plausible -448.
-    float c[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) c[j] = (v[j] != v[j]) ? v[j] : fminf(fmaxf(v[j], -448.f), 448.f);
-    int w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
+    // overflowed-to-NaN result into a plausible largest value.
+    const int w = pack4_f8<CT>(v[0], v[1], v[2], v[3]);
     uint8_t* cp = C + off_el;
     if (vec && nvalid >= 4) { *(uint32_t*)cp = (uint32_t)w; return; }
 #pragma unroll
@@ -1047,6 +1061,7 @@ __device__ __forceinline__ void epilogue(const GemmParams& p, const TileCtx& tc,
   }
   if constexpr (is_f8(T::DT)) {
     if (p.c_type == DT_FP8) { epilogue_t<T, DT_FP8>(p, tc, acc, li); return; }
+    if (p.c_type == DT_E5M2) { epilogue_t<T, DT_E5M2>(p, tc, acc, li); return; }
   }
   if (p.c_type == DT_BF16) epilogue_t<T, DT_BF16>(p, tc, acc, li);
   else if (p.c_type == DT_F16) epilogue_t<T, DT_F16>(p, tc, acc, li);

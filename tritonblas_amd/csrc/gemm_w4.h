@@ -130,16 +130,11 @@ __device__ __forceinline__ void epilogue_w4(const GemmParams& p, const TileCtx& 
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = v[e] + bv[e];
       }
-      if constexpr (CT == DT_FP8) {
-        // fp32 -> e4m3fn: clamp to the largest finite value (NaN stays NaN, as torch.clamp keeps it), round to
+      if constexpr (is_f8(CT)) {
+        // fp32 -> e4m3fn / e5m2: clamp to the largest finite value (NaN stays NaN, as torch.clamp keeps it), round to
         // nearest even; eight consecutive output columns are eight bytes
-        float cl[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) cl[e] = (v[e] != v[e]) ? v[e] : fminf(fmaxf(v[e], -448.f), 448.f);
-        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[0], cl[1], 0, false);
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[2], cl[3], w0, true);
-        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[4], cl[5], 0, false);
-        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(cl[6], cl[7], w1, true);
+        const int w0 = pack4_f8<CT>(v[0], v[1], v[2], v[3]);
+        const int w1 = pack4_f8<CT>(v[4], v[5], v[6], v[7]);
         uint8_t* cp = p.C + ((int64_t)m * p.c_sm + (int64_t)n * p.c_sn);
         if (p.c_vec && p.c_sn == 1 && nvalid >= 8 && (((uintptr_t)cp) & 7) == 0) {
           *(uint2*)cp = uint2{(uint32_t)w0, (uint32_t)w1};
@@ -573,6 +568,8 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
       else if (p.c_type == DT_F16) epilogue_w4<T, DT_F16>(p, w.tc, ln);
       else if (is_f8(T::DT) && p.c_type == DT_FP8) {
         if constexpr (is_f8(T::DT)) epilogue_w4<T, DT_FP8>(p, w.tc, ln);
+      } else if (is_f8(T::DT) && p.c_type == DT_E5M2) {
+        if constexpr (is_f8(T::DT)) epilogue_w4<T, DT_E5M2>(p, w.tc, ln);
       } else epilogue_w4<T, DT_F32>(p, w.tc, ln);
       nst = fast ? 1 : 0;
     }

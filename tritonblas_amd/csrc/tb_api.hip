@@ -188,7 +188,8 @@ int default_panel_n(int grid, int chunk, int group_m) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : (dt == TB_F32 ? 4 : 1); }
-int c_bytes(int t) { return t == TB_F32 ? 4 : ((t == TB_I8 || t == TB_FP8_E4M3) ? 1 : 2); }
+bool is_f8_type(int t) { return t == TB_FP8_E4M3 || t == TB_FP8_E5M2; }
+int c_bytes(int t) { return t == TB_F32 ? 4 : ((t == TB_I8 || is_f8_type(t)) ? 1 : 2); }
 
 // Everything the launch path needs, independent of which public descriptor it came from.
 struct Job {
@@ -248,7 +249,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
   if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
   if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8) &&
-      !(j.c_type == TB_FP8_E4M3 && (j.dt == TB_FP8_E4M3 || j.dt == TB_FP8_E5M2)))
+      !(is_f8_type(j.c_type) && is_f8_type(j.dt)))
     return TB_ERR_BAD_DTYPE;
   const int usz = unit_bytes(j.dt);
   const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
@@ -302,7 +303,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (is_streamk(j.schedule)) at_once = j.grid > 0 ? std::max<int64_t>(at_once, j.grid) : 0;
     if (j.num_groups > 0) at_once = 0;
     v = find_variant(j.dt, bm, bn, bk, alay, blay, 1, at_once, &hw, is_streamk(j.schedule) && j.num_groups == 0, j.K,
-                     j.c_type == TB_I8 ? 2 : (j.c_type == TB_FP8_E4M3 ? 1 : 0));
+                     j.c_type == TB_I8 ? 2 : (is_f8_type(j.c_type) ? 1 : 0));
     if (!v) return TB_ERR_BAD_TILE;
   } else {
     if (j.bm != 0) {
@@ -329,7 +330,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   p.a_vec = p.b_vec = v->fast;
   const int cb = c_bytes(j.c_type);
   p.c_vec = (j.c_sn == 1 && (j.c_sm % 4 == 0 || j.M == 1) && ((uintptr_t)j.C % (4 * cb)) == 0) ? 1 : 0;
-  p.c_line = (j.c_type != TB_I8 && j.c_type != TB_FP8_E4M3 && j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
+  p.c_line = (j.c_type != TB_I8 && !is_f8_type(j.c_type) && j.c_sn == 1 && ((j.c_sm * cb) % 16 == 0 || j.M == 1) && ((uintptr_t)j.C % 16) == 0) ? 1 : 0;
   if (hooks().no_cline) p.c_line = 0;
   // (8192x28672x8192 FP8 +0.6 %, 8192^3 bf16 +1.6 %; a small C stays cacheable for whoever reads it next)
   p.c_nt = ((int64_t)j.M * j.N * cb > (int64_t)hw.num_xcd * std::max(hw.l2_bytes, 1 << 20)) ? 1 : 0;
@@ -358,7 +359,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     // the model expects it to beat the tile kernel of the requested schedule.  TB_NO_SKINNY=1 / TB_SKINNY=1
     // force the choice (tuning and tests).
     plan->skinny = j.num_groups == 0 && skinny_supported(j.dt, j.M) && alay == LAY_K && blay == LAY_K &&
-                   KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !hooks().no_skinny && j.c_type != TB_FP8_E4M3;
+                   KU % skinny_k_step_units(j.dt) == 0 && j.N >= 1024 && !hooks().no_skinny && !is_f8_type(j.c_type);
     if (plan->skinny && !hooks().skinny) {
       tb_problem pr;
       std::memset(&pr, 0, sizeof(pr));
@@ -470,7 +471,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
         return make_plan(whole, hw, need_device, plan);
       }
       if (v->fast && j.c_type != TB_I8) {
-        const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K, j.c_type == TB_FP8_E4M3 ? 1 : 0);
+        const Variant* w = find_variant(j.dt, v->bm, v->bn, v->bk, v->alay, v->blay, 1, 0, &hw, false, j.K, is_f8_type(j.c_type) ? 1 : 0);
         if (w && w->k_step_pairs && w->bm == v->bm && w->bn == v->bn && w->bk == v->bk &&
             std::max(1, std::min(w->minb, hw.lds_bytes / w->lds_bytes)) == occ)
           v = w;
