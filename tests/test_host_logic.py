@@ -162,6 +162,36 @@ def test_argument_validation_without_a_gpu():
         _lib.check(_lib.TB_ERR_BAD_TILE)
 
 
+def test_grouped_descriptor_validation_and_workspace_size_without_a_gpu():
+    """The grouped entry point's checks that need no device, and the workspace a Stream-K tail asks for: the flags
+    and one fp32 256x256 partial tile per workgroup of a 256-CU grid when the 4-wave kernel can take it (K a
+    multiple of 512), nothing otherwise."""
+    from tritonblas_amd import _lib
+    lib = _lib.load()
+    g = _lib.tb_grouped_gemm_desc()
+    assert lib.tb_grouped_gemm_fp8(g, None) == _lib.TB_ERR_BAD_ARGUMENT    # struct_bytes not set
+    g.struct_bytes = C.sizeof(_lib.tb_grouped_gemm_desc)
+    assert lib.tb_grouped_gemm_fp8(g, None) == _lib.TB_ERR_NULL_POINTER
+    g.a = g.w = g.c = g.group_offsets = 256                                # (never dereferenced: the checks below fail first)
+    g.c_type = _lib.TB_BF16
+    g.m_total, g.n, g.k, g.num_groups = 8192, 14336, 4096, 8
+    g.a_stride_m, g.w_stride_g, g.w_stride_n, g.c_stride_m, g.c_stride_n = 4096, 14336 * 4096, 4096, 14336, 1
+    g.streamk = 2
+    assert lib.tb_grouped_gemm_fp8(g, None) == _lib.TB_ERR_BAD_ARGUMENT
+    g.streamk = 0
+    g.small_rows = -2
+    assert lib.tb_grouped_gemm_fp8(g, None) == _lib.TB_ERR_BAD_ARGUMENT
+    g.small_rows = -1
+    assert lib.tb_grouped_workspace_bytes(g) == 0                          # no Stream-K tail asked for
+    g.streamk = 1
+    _, flags_off = _lib.workspace_layout()
+    assert lib.tb_grouped_workspace_bytes(g) == flags_off + 1024 + 256 * 256 * 256 * 4
+    g.k = 4096 + 128                                                       # an odd number of K steps: 8-wave kernel, whole tiles
+    g.a_stride_m = g.w_stride_n = g.k
+    g.w_stride_g = 14336 * g.k
+    assert lib.tb_grouped_workspace_bytes(g) == 0
+
+
 def test_python_api_refuses_cpu_tensors():
     import tritonblas_amd as tb
     a = torch.zeros(16, 16, dtype=torch.float16)
