@@ -44,8 +44,9 @@ enum {
   TB_F32 = 4,       /* operands (full fp32 products, 16x16x4 MFMA), output, bias, quantiser input */
   TB_I8 = 5,        /* operands (int32 sums, persistent_gemm.py:75); as output only with TB_I8 operands: fp32 epilogue
                        result truncated toward zero and saturated to [-128, 127]                    */
-  TB_FP8_E5M2 = 6   /* OCP e5m2, operands of tb_gemm only (the type utils.py:46 lists next to e4m3); both
-                       operands must have the same 8-bit format                                     */
+  TB_FP8_E5M2 = 6   /* OCP e5m2, operands of tb_gemm only (the type utils.py:46 lists next to e4m3); one operand may be
+                       e4m3 and the other e5m2 (origami.py:98-112 takes a_dtype and b_dtype separately) -- the only
+                       pair of different operand types tb_gemm accepts                               */
 };
 /* TB_FP8_E4M3 and TB_FP8_E5M2 are also accepted as the OUTPUT type of a GEMM with TB_FP8_E4M3 or TB_FP8_E5M2 operands:
  * the fp32 epilogue result is clamped to the format's largest finite value (+-448, +-57344; NaN stays NaN) and rounded

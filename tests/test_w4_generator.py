@@ -4,6 +4,7 @@ workgroup, after compiled epilogue stores, after a fused epilogue) and must not 
 in flight than were issued after the copies it waits for."""
 import importlib.util
 import os
+import re
 
 import pytest
 
@@ -18,7 +19,7 @@ def _load():
     return mod
 
 
-@pytest.mark.parametrize("kind", ["fp8", "e5m2", "fp4", "bf16", "f16", "i8"])
+@pytest.mark.parametrize("kind", ["fp8", "e5m2", "e4e5", "e5e4", "fp4", "bf16", "f16", "i8"])
 def test_wait_counts_hold_for_every_history(kind):
     gen = _load()
     slack = gen.Gen(kind).check()
@@ -64,12 +65,16 @@ def test_program_shape(kind):
     assert all(t.count("a[") == 2 for t in steady)
 
 
-def test_e5m2_differs_from_e4m3_only_in_the_format_field():
+@pytest.mark.parametrize("kind,fields", [("e5m2", " cbsz:1 blgp:1"), ("e4e5", " cbsz:1"), ("e5e4", " blgp:1")])
+def test_8bit_float_kinds_differ_from_e4m3_only_in_the_format_fields(kind, fields):
+    """cbsz is the format of the MFMA's first source, which is the B fragment, blgp that of the second, the A
+    fragment: e4e5 (A in e4m3, B in e5m2) sets cbsz alone, e5e4 blgp alone."""
     gen = _load()
-    a, b = gen.Gen("fp8").program(), gen.Gen("e5m2").program()
+    a, b = gen.Gen("fp8").program(), gen.Gen(kind).program()
     assert len(a) == len(b)
     for x, y in zip(a, b):
         if x.startswith("v_mfma"):
-            assert y == x + " cbsz:1 blgp:1"
+            assert y == x + fields
+            assert re.match(r"v_mfma_f32_16x16x128_f8f6f4 a\[\d+:\d+\], v\[(\d+):\d+\], v\[(\d+):\d+\]", x)
         else:
             assert x == y

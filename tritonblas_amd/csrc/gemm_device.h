@@ -18,9 +18,14 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 
-enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4, DT_I8 = 5, DT_E5M2 = 6 };
-// the two 8-bit float formats (OCP e4m3 = DT_FP8, e5m2) share everything but the MFMA's format field
-constexpr bool is_f8(int dt) { return dt == DT_FP8 || dt == DT_E5M2; }
+enum : int { DT_F16 = 0, DT_BF16 = 1, DT_FP8 = 2, DT_FP4 = 3, DT_F32 = 4, DT_I8 = 5, DT_E5M2 = 6,
+             DT_E4E5 = 7,    // A in e4m3, B in e5m2 (operand types only; never an output type)
+             DT_E5E4 = 8 };  // A in e5m2, B in e4m3
+// the two 8-bit float formats (OCP e4m3 = DT_FP8, e5m2) and their two mixtures share everything but the
+// MFMA's format fields (0 = e4m3, 1 = e5m2, one field per operand)
+constexpr bool is_f8(int dt) { return dt == DT_FP8 || dt == DT_E5M2 || dt == DT_E4E5 || dt == DT_E5E4; }
+constexpr int f8_fmt_a(int dt) { return (dt == DT_E5M2 || dt == DT_E5E4) ? 1 : 0; }
+constexpr int f8_fmt_b(int dt) { return (dt == DT_E5M2 || dt == DT_E4E5) ? 1 : 0; }
 enum : int { MODE_STATIC = 0, MODE_WS = 1, MODE_SK = 2, MODE_GROUPED = 3 };
 enum : int { WS_QUEUES = 0, WS_GLOBAL = 1, WS_HIERARCHICAL = 2 };   // how work-stealing workgroups find tiles
 enum : int { LAY_K = 0, LAY_M = 1 };  // which index is contiguous in global memory for an operand
@@ -454,8 +459,8 @@ __device__ __forceinline__ v4f mma(typename Frag<T>::type x, typename Frag<T>::t
     // exact int32 sums: the accumulator registers hold integers until the K loop ends
     return __builtin_bit_cast(v4f, __builtin_amdgcn_mfma_i32_16x16x64_i8(x, y, __builtin_bit_cast(v4i, c), 0, 0, 0));
   } else if constexpr (is_f8(T::DT)) {
-    constexpr int FMT = T::DT == DT_E5M2 ? 1 : 0;   // format field of both operands: 0 = e4m3, 1 = e5m2
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, FMT, FMT, 0, 0, 0, 0);
+    // (x is the B fragment, y the A fragment: the first format field is B's)
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, f8_fmt_b(T::DT), f8_fmt_a(T::DT), 0, 0, 0, 0);
   } else {
     v8i x8 = {x.x, x.y, x.z, x.w, 0, 0, 0, 0};
     v8i y8 = {y.x, y.y, y.z, y.w, 0, 0, 0, 0};

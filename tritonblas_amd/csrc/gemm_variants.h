@@ -47,6 +47,10 @@ extern const Variant g_variants_fp8[];
 extern const int g_num_variants_fp8;
 extern const Variant g_variants_e5m2[];
 extern const int g_num_variants_e5m2;
+extern const Variant g_variants_e4e5[];
+extern const int g_num_variants_e4e5;
+extern const Variant g_variants_e5e4[];
+extern const int g_num_variants_e5e4;
 extern const Variant g_variants_fp4[];
 extern const int g_num_variants_fp4;
 extern const Variant g_variants_f32[];

@@ -343,8 +343,9 @@ __device__ __forceinline__ void epilogue_w4_owner(const GemmParams& p, const Til
       [cprev] "s"(s_cprev), [cstep] "s"(s_cstep)
 
 #ifdef W4_LAB_TS
-// measurement build: when (constant 100 MHz counter) every workgroup started and finished each of its tiles
-__device__ unsigned long long w4_lab_ts[1024 * 32];
+// measurement build: when (constant 100 MHz counter) every workgroup started and finished each of its tiles (one array per
+// translation unit that includes this file; the one the host reads back is that of the 8-bit float kernels)
+static __device__ unsigned long long w4_lab_ts[1024 * 32];
 #endif
 
 // SK: the schedule may end in a Stream-K tail (pieces of a tile's K range, cut at multiples of four K steps:
@@ -464,6 +465,22 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
             : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
             :
 #include "w4_clobbers_e5m2.inc"
+        );
+      } else if constexpr (T::DT == DT_E4E5) {
+        asm volatile(
+#include "w4_kloop_e4e5.inc"
+            : [scbuf] "+s"(scbuf)
+            : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
+            :
+#include "w4_clobbers_e4e5.inc"
+        );
+      } else if constexpr (T::DT == DT_E5E4) {
+        asm volatile(
+#include "w4_kloop_e5e4.inc"
+            : [scbuf] "+s"(scbuf)
+            : W4_COMMON_OPERANDS, [eo] "{v[240:243]}"(eo), [sap] "s"(s_sap), [sbp] "s"(s_sbp)
+            :
+#include "w4_clobbers_e5e4.inc"
         );
       } else {
         asm volatile(

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Writes the hand-scheduled K loop of the 4-wave 256x256 tile kernels (gemm_w4.h) as inline-assembly text.
 
-    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: e5m2, fp4, bf16, f16, i8)
+    python3 gen_w4.py fp8 > w4_kloop_fp8.inc        (also: e5m2, e4e5, e5e4, fp4, bf16, f16, i8)
     python3 gen_w4.py clobbers fp8 > w4_clobbers_fp8.inc
     python3 gen_w4.py check                          (walks every kind through the wait-count checker)
 
@@ -93,12 +93,17 @@ class WaitVm:
         self.awaits, self.vals = awaits, {k: (None if v is None else min(63, v)) for k, v in vals.items()}
 
 
+F8_KINDS = ("fp8", "e5m2", "e4e5", "e5e4")
+
+
 class Gen:
     def __init__(self, kind, lab=()):
-        self.kind = kind                # "fp8" | "e5m2" | "fp4" | "bf16" | "f16" | "i8"
-        self.f8 = kind in ("fp8", "e5m2")   # 8-bit floats: one MFMA of K = 128 per fragment pair; they differ in its format field
+        self.kind = kind                # "fp8" | "e5m2" | "e4e5" | "e5e4" | "fp4" | "bf16" | "f16" | "i8"
+        # 8-bit floats: one MFMA of K = 128 per fragment pair; the kinds differ in its format fields (e4e5: A in e4m3, B in
+        # e5m2; e5e4 the other way round)
+        self.f8 = kind in F8_KINDS
         self.fp4 = kind == "fp4"        # (the only kind with E8M0 scale operands)
-        self.scaled_epi = kind in ("fp8", "e5m2", "i8")  # the fused epilogue multiplies by sa[m] * sb[n]
+        self.scaled_epi = kind in F8_KINDS or kind == "i8"  # the fused epilogue multiplies by sa[m] * sb[n]
         self.int_acc = kind == "i8"      # int32 sums: converted to fp32 where they leave the accumulators
         self.nm = 8 if self.f8 else 16      # MFMAs per row block (FP8: one of K = 128 per fragment pair; others: two half-K ones)
         self.nsc = 4 if self.scaled_epi else 0    # copies of the tile's own epilogue scales (step 1)
@@ -190,7 +195,8 @@ class Gen:
             acc = (i * 8 + j) * 4
             b, a = self.vB(p, j), self.vA(i)
             c = "0" if zero else f"a[{acc}:{acc + 3}]"
-            fmt = " cbsz:1 blgp:1" if self.kind == "e5m2" else ""      # (format of both operands; e4m3 is the default)
+            # format fields: cbsz = the first source (the B fragment), blgp = the second (the A fragment); e4m3 is the default
+            fmt = {"fp8": "", "e5m2": " cbsz:1 blgp:1", "e4e5": " cbsz:1", "e5e4": " blgp:1"}[self.kind]
             return Op(f"v_mfma_f32_16x16x128_f8f6f4 a[{acc}:{acc + 3}], v[{b}:{b + 7}], v[{a}:{a + 7}], {c}{fmt}")
         # two MFMAs per accumulator and K step, k slice outermost so that the same accumulator comes up
         # again only eight instructions later
@@ -686,7 +692,7 @@ def main():
         sys.stdout.write(clobbers(sys.argv[2]))
         return
     if what == "check":
-        for kind in ("fp8", "e5m2", "fp4", "bf16", "f16", "i8"):
+        for kind in F8_KINDS + ("fp4", "bf16", "f16", "i8"):
             w = Gen(kind).check()
             print(kind, "ok; smallest slack per wait site:", min(w.values()), "largest:", max(w.values()))
         return

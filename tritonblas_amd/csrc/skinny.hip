@@ -148,7 +148,11 @@ static hipError_t launch_dt(const GemmParams& p, hipStream_t stream) {
   return launch_mt<DT, 4>(p, stream);
 }
 
-bool skinny_supported(int dt, int64_t m) { return m <= SKINNY_MAX_M && (is_f8(dt) || dt == DT_F16 || dt == DT_BF16); }
+// (operands of two different 8-bit float formats stay on the tile kernels: this compiler crashes on a translation unit
+// that holds MFMAs of both mixtures, and a streaming kernel per mixture in files of their own is not worth two more)
+bool skinny_supported(int dt, int64_t m) {
+  return m <= SKINNY_MAX_M && (dt == DT_FP8 || dt == DT_E5M2 || dt == DT_F16 || dt == DT_BF16);
+}
 
 int skinny_k_step_units(int dt) { return is_f8(dt) ? 128 : 32; }
 

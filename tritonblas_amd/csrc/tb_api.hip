@@ -122,6 +122,8 @@ void variant_table(int dt, const Variant** v, int* n) {
     case TB_BF16: *v = g_variants_bf16; *n = g_num_variants_bf16; break;
     case TB_FP8_E4M3: *v = g_variants_fp8; *n = g_num_variants_fp8; break;
     case TB_FP8_E5M2: *v = g_variants_e5m2; *n = g_num_variants_e5m2; break;
+    case DT_E4E5: *v = g_variants_e4e5; *n = g_num_variants_e4e5; break;
+    case DT_E5E4: *v = g_variants_e5e4; *n = g_num_variants_e5e4; break;
     case TB_FP4_E2M1: *v = g_variants_fp4; *n = g_num_variants_fp4; break;
     case TB_F32: *v = g_variants_f32; *n = g_num_variants_f32; break;
     case TB_I8: *v = g_variants_i8; *n = g_num_variants_i8; break;
@@ -189,6 +191,17 @@ int default_panel_n(int grid, int chunk, int group_m) {
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 int unit_bytes(int dt) { return (dt == TB_F16 || dt == TB_BF16) ? 2 : (dt == TB_F32 ? 4 : 1); }
 bool is_f8_type(int t) { return t == TB_FP8_E4M3 || t == TB_FP8_E5M2; }
+// The kernels' element type code for a pair of operand types: the type itself when both agree, the codes of the two
+// mixtures of 8-bit float formats (reference origami.py:98-112 and matmul.py:42-66 take the two types separately), -1 for
+// any other pair.
+int kernel_type(int a_type, int b_type) {
+  if (a_type == b_type) return a_type;
+  if (a_type == TB_FP8_E4M3 && b_type == TB_FP8_E5M2) return DT_E4E5;
+  if (a_type == TB_FP8_E5M2 && b_type == TB_FP8_E4M3) return DT_E5E4;
+  return -1;
+}
+// the type the cost model prices a kernel type as (the mixtures run the e5m2 kernels' instruction stream)
+int model_type(int dt) { return (dt == DT_E4E5 || dt == DT_E5E4) ? TB_FP8_E5M2 : dt; }
 int c_bytes(int t) { return t == TB_F32 ? 4 : ((t == TB_I8 || is_f8_type(t)) ? 1 : 2); }
 
 // Everything the launch path needs, independent of which public descriptor it came from.
@@ -249,7 +262,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (j.M <= 0 || j.N <= 0 || j.K <= 0) return TB_ERR_BAD_SHAPE;
   if (j.M > INT32_MAX || j.N > INT32_MAX) return TB_ERR_BAD_SHAPE;
   if (j.c_type != TB_F16 && j.c_type != TB_BF16 && j.c_type != TB_F32 && !(j.c_type == TB_I8 && j.dt == TB_I8) &&
-      !(is_f8_type(j.c_type) && is_f8_type(j.dt)))
+      !(is_f8_type(j.c_type) && is_f8(j.dt)))
     return TB_ERR_BAD_DTYPE;
   const int usz = unit_bytes(j.dt);
   const int epu = (j.dt == TB_FP4_E2M1) ? 2 : 1;
@@ -274,7 +287,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
   if (bm == 0 || bn == 0 || bk == 0) {
     tb_problem pr;
     std::memset(&pr, 0, sizeof(pr));
-    pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+    pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = model_type(j.dt); pr.c_type = j.c_type;
     pr.a_k_contiguous = alay == LAY_K; pr.b_k_contiguous = blay == LAY_K;
     pr.streamk = is_streamk(j.schedule); pr.num_groups = j.num_groups;
     auto infos = tile_infos(j.dt);
@@ -363,7 +376,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (plan->skinny && !hooks().skinny) {
       tb_problem pr;
       std::memset(&pr, 0, sizeof(pr));
-      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = model_type(j.dt); pr.c_type = j.c_type;
       pr.a_k_contiguous = pr.b_k_contiguous = 1;
       const bool sk = is_streamk(j.schedule);
       const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, v->minb, v->fast, v->stages};
@@ -443,7 +456,7 @@ int make_plan(const Job& j, const tb_hw& hw, bool need_device, Plan* plan) {
     if (g <= 0 || g > resident) {
       tb_problem pr;
       std::memset(&pr, 0, sizeof(pr));
-      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+      pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = model_type(j.dt); pr.c_type = j.c_type;
       pr.a_k_contiguous = pr.b_k_contiguous = 1; pr.streamk = 1;
       tb_hw hw_res = hw;   // (what the model may fill: the kernel's real occupancy)
       const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, occ, v->fast, v->stages};
@@ -624,7 +637,7 @@ int64_t column_split_point(const Job& j, const tb_hw& hw, const Plan& whole) {
   const int64_t n1 = tn1 * v->bn, n2 = j.N - n1;
   tb_problem pr;
   std::memset(&pr, 0, sizeof(pr));
-  pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = j.dt; pr.c_type = j.c_type;
+  pr.m = j.M; pr.n = j.N; pr.k = j.K; pr.a_type = pr.b_type = model_type(j.dt); pr.c_type = j.c_type;
   pr.a_k_contiguous = pr.b_k_contiguous = 1;
   const TileInfo ti{v->dt, v->bm, v->bn, v->bk, v->threads, v->lds_bytes, v->minb, v->fast, v->stages};
   const double t_whole = estimate_tile_us(pr, hw, ti, false);
@@ -712,13 +725,14 @@ void init_scratch(int dev) {
 int job_from_gemm(const tb_gemm_desc* d, Job* j) {
   if (!d) return TB_ERR_NULL_POINTER;
   if (d->struct_bytes != sizeof(tb_gemm_desc)) return TB_ERR_BAD_ARGUMENT;
-  if (d->a_type != d->b_type) return TB_ERR_BAD_DTYPE;
   if (d->a_type != TB_F16 && d->a_type != TB_BF16 && d->a_type != TB_FP8_E4M3 && d->a_type != TB_FP8_E5M2 && d->a_type != TB_F32 &&
       d->a_type != TB_I8)
     return TB_ERR_BAD_DTYPE;
+  const int dt = kernel_type(d->a_type, d->b_type);
+  if (dt < 0) return TB_ERR_BAD_DTYPE;
   if ((d->a_scale == nullptr) != (d->b_scale == nullptr)) return TB_ERR_BAD_ARGUMENT;
   if (d->bias && d->bias_type != TB_F16 && d->bias_type != TB_BF16 && d->bias_type != TB_F32) return TB_ERR_BAD_DTYPE;
-  j->dt = d->a_type; j->c_type = d->c_type; j->bias_type = d->bias_type;
+  j->dt = dt; j->c_type = d->c_type; j->bias_type = d->bias_type;
   j->M = d->m; j->N = d->n; j->K = d->k;
   j->A = d->a; j->B = d->b; j->C = d->c;
   j->a_sr = d->a_stride_m; j->a_sk = d->a_stride_k; j->b_sr = d->b_stride_n; j->b_sk = d->b_stride_k;
@@ -844,9 +858,13 @@ int tb_select(const tb_problem* problem, const tb_hw* hw, tb_selection* out) {
   if (problem->m <= 0 || problem->n <= 0 || problem->k <= 0) return TB_ERR_BAD_SHAPE;
   tb_hw local;
   if (hw) local = *hw; else default_hw(&local);
-  auto infos = tile_infos(problem->a_type);
+  const int dt = kernel_type(problem->a_type, problem->b_type);
+  if (dt < 0) return TB_ERR_BAD_DTYPE;
+  auto infos = tile_infos(dt);
   if (infos.empty()) return TB_ERR_BAD_DTYPE;
-  return select_tile(*problem, local, infos.data(), (int)infos.size(), out);
+  tb_problem pr = *problem;
+  pr.a_type = pr.b_type = model_type(dt);
+  return select_tile(pr, local, infos.data(), (int)infos.size(), out);
 }
 
 int tb_gemm(const tb_gemm_desc* desc, void* stream) {
