@@ -74,10 +74,18 @@ int variant_occupancy(const TileInfo& v, const tb_hw& hw) {
 //     time its own copy takes at the ~100 GB/s one workgroup pulls (0.46 us for a 16 KB step, 0.65 us
 //     for 40 KB): small problems want enough tiles to put several workgroups on every CU, and
 //     long-K problems with few rows want the deep 32x128x256 tile;
-//   * per tile: epilogue + first-copy latency, ~12 us for 256x256, ~4 us for 128x128, ~3 us below.
-static double family_efficiency(int dt, const TileInfo& v) {
+//   * per tile: epilogue + first-copy latency, ~12 us for 256x256 (8 us on the 4-wave kernel), ~4 us for 128x128, ~3 us below.
+// w4: the hand-scheduled 4-wave kernel runs the 256x256 tile (K an even number of K steps, at least four); its
+// figures are from rounds of 256 tiles at K = 4096 and 8192 (FP8 46.5 and 85.7 us per round, bf16 89 and 178 us,
+// MXFP4 8192x8192x16384 in 0.40-0.43 ms) with 8 us per tile.
+static double family_efficiency(int dt, const TileInfo& v, bool w4) {
   const int area = v.bm * v.bn;
   const int cls = (v.bm < 64 || v.bn < 64) ? 3 : (area >= 256 * 256 ? 0 : (area >= 128 * 128 ? 1 : 2));
+  if (w4 && cls == 0) {
+    if (dt == TB_FP8_E4M3 || dt == TB_FP8_E5M2 || dt == TB_I8) return 0.705;
+    if (dt == TB_FP4_E2M1) return 0.56;
+    if (dt == TB_F16 || dt == TB_BF16) return 0.655;
+  }
   static const double f8[4] = {0.61, 0.46, 0.29, 0.15};     // (128x128: 8192x28672x8192 in 1.72-1.77 ms, 8192^3 in 0.48 ms)
   static const double h16[4] = {0.59, 0.465, 0.22, 0.12};  // (128x128: 8192^3 bf16 in 0.97 ms)
   static const double f4[4] = {0.50, 0.36, 0.22, 0.10};     // (256x256: the 4-wave kernel, 8192x8192x16384 in 0.43-0.47 ms)
@@ -102,8 +110,27 @@ static double family_efficiency(int dt, const TileInfo& v) {
 //     unless another round of whole tiles is expected to be as fast (large tiles have expensive partial
 //     tiles: 2048x14336x4096 bf16, 448 tiles of 256x256 on 256 slots: 209 us in two rounds, 253 us with a
 //     shared tail); the return value `total` means "whole tiles only".
+// A last round that does not fill the CUs is cheaper than a full one for the 256x256 tiles (one workgroup per CU):
+// the busy CUs run at a higher clock and share the L2s and the fabric with fewer others.  Measured, FP8 and bf16,
+// K = 4096 and 8192, as a fraction of a full round: 0.66-0.69 with 6 % of the CUs busy, 0.84-0.91 with a quarter,
+// 0.87-0.93 with half or three quarters.  f: the busy fraction.
+static double partial_round_factor(double f) {
+  if (f <= 0.0 || f >= 1.0) return 1.0;
+  return f < 0.25 ? 0.65 + f : (f < 0.75 ? 0.9 : 0.9 + 0.4 * (f - 0.75));
+}
 static const double kSharedTailFactor = 4.0;
-int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us) {
+// What the exchange of partial tiles costs the workgroup that finishes a tile cut into `segments` pieces, when
+// `partials` partial tiles are exchanged at about the same time.  xchg_us = 0 (the 8-wave kernels): fix_us per extra
+// piece, one after the other, times `crowd` when a whole grid shares a tail.  xchg_us > 0 (the 4-wave 256x256 kernels,
+// whose pieces exchange 256 KB each): the exchange is bound by what all of them move together -- 128 tiles cut in two
+// 30 us, 64 tiles cut in four 43 us, a tail of 280 tiles shared by 256 workgroups 60 us: 0.23 us per partial tile,
+// about 1.1 TB/s -- and never faster than one workgroup reads its partners' tiles (fix_us each).
+static double exchange_us(double segments, double partials, double fix_us, double xchg_us, double crowd) {
+  if (segments <= 1.0) return 0.0;
+  if (xchg_us > 0.0) return std::max((segments - 1.0) * fix_us, partials * xchg_us);
+  return (segments - 1.0) * fix_us * crowd;
+}
+int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us, double xchg_us) {
   if (total <= 0 || slots <= 0) return 1;
   if (total >= slots) {
     const int64_t tail = total % slots;
@@ -111,8 +138,10 @@ int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double ste
     // (a tail shared by the whole grid costs about four times the per-segment figure that the split of
     // a few tiles shows: 2048x28672x8192 FP8, 128 tiles of 256x256 shared by 256 workgroups, ~100 us on
     // top of their K steps; 1024x28672x8192, 192 shared tiles, the same)
-    const double shared = std::ceil((double)tail * k_iters / slots) * step_us + (std::ceil((double)slots / tail) - 1.0) * fix_us * kSharedTailFactor;
-    const double whole = (double)k_iters * step_us;
+    const double segments = std::ceil((double)slots / tail);
+    const double shared = std::ceil((double)tail * k_iters / slots) * step_us +
+                          exchange_us(segments, (double)(slots - tail), fix_us, xchg_us, kSharedTailFactor);
+    const double whole = (double)k_iters * step_us * (xchg_us > 0.0 ? partial_round_factor((double)tail / slots) : 1.0);
     return shared < whole ? slots : (int)std::min<int64_t>(total, INT32_MAX);
   }
   if (total >= n_cu) return (int)total;
@@ -122,7 +151,8 @@ int streamk_grid(int64_t total, int64_t k_iters, int slots, int n_cu, double ste
   for (int64_t s2 = 1; s2 <= smax && (s2 == 1 || k_iters / s2 >= 8); s2 *= 2) {
     // workgroups per CU grow with the split; beyond one per CU they share its matrix pipe
     const double share = std::max(1.0, (double)(total * s2) / n_cu);
-    const double cost = std::ceil((double)k_iters / s2) * step_us * std::sqrt(share) + (s2 - 1) * fix_us;
+    const double cost = std::ceil((double)k_iters / s2) * step_us * std::sqrt(share) +
+                        exchange_us((double)s2, (double)(total * (s2 - 1)), fix_us, xchg_us, 1.0);
     if (s2 == 1 || cost < best) { best = cost; best_s = s2; }
   }
   return (int)(total * best_s);
@@ -140,7 +170,8 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   const int area = v.bm * v.bn;
 
   const double ideal_step_us = 2.0 * v.bm * v.bn * v.bk / mfma_flops_per_clk(pr.a_type) / clk * 1e6;
-  const double t_thru = ideal_step_us / family_efficiency(pr.a_type, v);   // CU time per tile K step, saturated
+  const bool w4 = v.threads == 256 && area >= 256 * 256 && k_iters >= 4 && k_iters % 2 == 0;
+  const double t_thru = ideal_step_us / family_efficiency(pr.a_type, v, w4);   // CU time per tile K step, saturated
   double t_lat = 0.30 + (v.bm + v.bn) * (v.bk * esz) / 1.0e5;                // floor per K step of one workgroup: round trip + its own copy at ~100 GB/s
   // the 64x64 tile of the 8- and 16-bit float types runs with four (three) copy stages while no more
   // than two (three) tiles per CU exist, which hides that much more of the round trip (measured x0.67 / x0.85)
@@ -154,7 +185,12 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
   if (v.bm == 128 && v.bn == 128 && pr.num_groups == 0 && pr.a_type == TB_FP8_E4M3 &&
       cdiv(pr.m, v.bm) * cdiv(pr.n, v.bn) <= (int64_t)hw.n_cu)
     t_lat *= 0.67;
-  const double t_tile = area >= 256 * 256 ? 12.0 : (area >= 128 * 128 ? 4.0 : 3.0);
+  const double t_tile = area >= 256 * 256 ? (w4 ? 8.0 : 12.0) : (area >= 128 * 128 ? 4.0 : 3.0);
+  auto last_round = [&](int64_t n_tiles, int64_t per_round) {
+    const int64_t r = n_tiles % per_round;
+    if (r == 0 || area < 256 * 256) return 1.0;
+    return partial_round_factor((double)r / per_round);
+  };
 
   double us;
   if (streamk) {
@@ -162,16 +198,19 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
     // owner, one after the other: ~1.5 us + the fp32 tile at ~10 GB/s (fitted on segment-count sweeps:
     // 32x128 tiles ~3 us, 128x128 tiles ~8 us, 256x256 tiles ~30 us per extra segment)
     // The 4-wave 256x256 kernels (256 threads) exchange partial tiles straight from the accumulators with 16 loads in
-    // flight per lane: ~12 us per extra segment (fitted: 2048x2048x16384 cut in four, FP8 92 us, bf16 137 us).
-    const double fix_us = 1.5 + area * 4.0 / 10e3 * ((v.threads == 256 && area >= 256 * 256) ? 0.4 : 1.0);
+    // flight per lane: 4.5 us per partner for one workgroup alone, and 0.23 us per partial tile of the whole launch
+    // (see exchange_us).
+    const bool big4 = w4 && k_iters % 4 == 0;   // (the 4-wave Stream-K kernel cuts K at multiples of four steps)
+    const double fix_us = big4 ? 4.5 : 1.5 + area * 4.0 / 10e3;
+    const double xchg_us = big4 ? 0.23 : 0.0;
     const int slots = hw.n_cu * occ;
-    const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu, std::max(t_thru, t_lat), fix_us);
+    const int grid = streamk_grid(tiles, k_iters, slots, hw.n_cu, std::max(t_thru, t_lat), fix_us, xchg_us);
     if (sk_grid_out) *sk_grid_out = grid;
     const int launched = (int)std::min<int64_t>(grid, slots);     // (grid == tiles > slots: whole tiles, resident grid loops)
     const double w = (double)cdiv(launched, hw.n_cu);             // workgroups sharing the busiest CU
     const double t_step = std::max(w * t_thru, t_lat);
     if (grid >= tiles && tiles > slots) {
-      us = (double)cdiv(tiles, slots) * (k_iters * t_step + t_tile);
+      us = ((double)(cdiv(tiles, slots) - 1) + last_round(tiles, slots)) * (k_iters * t_step + t_tile);
     } else {
       const int64_t dp_rounds = tiles / grid, tail = tiles % grid;
       us = (double)dp_rounds * (k_iters * t_step + t_tile);
@@ -179,7 +218,8 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
         const double iters = std::ceil((double)tail * k_iters / grid);
         const double segments = std::ceil((double)grid / tail);
         // (tiles < grid: every tile is cut into `segments` pieces; otherwise a tail shared by the whole grid)
-        us += iters * t_step + (segments - 1.0) * fix_us * (dp_rounds > 0 ? kSharedTailFactor : 1.0) + t_tile;
+        const double partials = dp_rounds > 0 ? (double)(grid - tail) : (double)tail * (segments - 1.0);
+        us += iters * t_step + exchange_us(segments, partials, fix_us, xchg_us, dp_rounds > 0 ? kSharedTailFactor : 1.0) + t_tile;
       }
     }
   } else {
@@ -188,6 +228,7 @@ static double score(const tb_problem& pr, const tb_hw& hw, const TileInfo& v, bo
     const int64_t full = c / occ, rem = c % occ;
     us = (double)full * (k_iters * std::max(occ * t_thru, t_lat) + t_tile);
     if (rem) us += k_iters * std::max((double)rem * t_thru, t_lat) + t_tile;
+    if (occ == 1 && c > 1) us -= (1.0 - last_round(tiles, hw.n_cu)) * (k_iters * std::max(t_thru, t_lat) + t_tile);
   }
   *comp_us = us;
 

@@ -10,7 +10,7 @@ struct TileInfo {
 };
 
 void default_hw(tb_hw* hw);
-int streamk_grid(int64_t total_tiles, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us);
+int streamk_grid(int64_t total_tiles, int64_t k_iters, int slots, int n_cu, double step_us, double fix_us, double xchg_us = 0.0);
 // the Stream-K grid the model picks for one tile variant on a problem
 int streamk_grid_for(const tb_problem& pr, const tb_hw& hw, const TileInfo& v);
 int ws_counters_per_xcd(int64_t total_tiles);

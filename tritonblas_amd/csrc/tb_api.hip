@@ -653,6 +653,23 @@ int64_t column_split_point(const Job& j, const tb_hw& hw, const Plan& whole) {
 }
 
 int launch_columns(const Job& j, hipStream_t stream) {
+  if (j.schedule == TB_SCHED_STREAMK && j.column_split == 0 && j.num_groups == 0 && !hooks().no_column_split) {
+    // A Stream-K launch whose plan shares no tile runs whole tiles on the whole-tile kernel; it is then the
+    // persistent launch of the same tile, partial last round and all, and is treated as one.
+    tb_hw hw;
+    int st = current_hw(&hw);
+    if (st != TB_OK) return st;
+    Plan plan;
+    st = cached_plan(j, hw, &plan);
+    if (st != TB_OK) return st;
+    if (plan.skinny || plan.p.mode != MODE_STATIC) return run_plan(j, plan, stream);
+    Job whole = j;
+    whole.schedule = TB_SCHED_PERSISTENT;
+    whole.grid = 0;
+    whole.bm = plan.v->bm; whole.bn = plan.v->bn; whole.bk = plan.v->bk;
+    whole.workspace = nullptr; whole.workspace_bytes = 0;
+    return launch_columns(whole, stream);
+  }
   if (j.schedule != TB_SCHED_PERSISTENT || j.column_split != 0 || j.grid > 0 || j.num_groups > 0 || hooks().no_column_split)
     return launch(j, stream);
   tb_hw hw;
