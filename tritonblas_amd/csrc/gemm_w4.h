@@ -446,6 +446,11 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
     const int s_kh = uniform(kh), s_first = uniform(first), s_nst = uniform(nst), s_fe = uniform(fe);
     const uint8_t* s_cprev = uniform(cprev);
     scbuf = uniform(scbuf);
+#ifdef W4_LAB_TS2
+    // (with -DW4_LAB_TS -DW4_LAB_TS2: two stamps per tile, in front of and behind its K loop statement, instead of one)
+    if (tid == 0 && blockIdx.x < 1024 && ts_n < 31) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
+    ++ts_n;
+#endif
     if constexpr (is_f8(T::DT) || T::DT == DT_I8) {
       // (a tile without scales or off the fast path loads 512 bytes of its operands instead; nobody uses them)
       const uint8_t* s_sap = uniform(regs ? (const uint8_t*)(p.sa + w.tc.m0 + ln.wm0) : cur.A);
@@ -521,6 +526,10 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
 #include "w4_clobbers_fp4.inc"
       );
     }
+#ifdef W4_LAB_TS2
+    if (tid == 0 && blockIdx.x < 1024 && ts_n < 31) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
+    ++ts_n;
+#endif
     bool sk_piece = false;
     if constexpr (SK) {
       if (w.kind == WK_SK_PUBLISH) {
@@ -590,7 +599,7 @@ __global__ __launch_bounds__(256, 1) void gemm_kernel_w4(const GemmParams p) {
       } else epilogue_w4<T, DT_F32>(p, w.tc, ln);
       nst = fast ? 1 : 0;
     }
-#ifdef W4_LAB_TS
+#if defined(W4_LAB_TS) && !defined(W4_LAB_TS2)
     if (tid == 0 && blockIdx.x < 1024 && ts_n < 31) w4_lab_ts[blockIdx.x * 32 + ts_n] = __builtin_amdgcn_s_memrealtime();
     ++ts_n;
 #endif
